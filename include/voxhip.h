@@ -353,6 +353,69 @@ int vox_lm_prefill(vox_lm* m, void* stream, const vox_lm_io* io, const int32_t* 
                    const void* row_features, const int32_t* q_req, int n_rows, const int32_t* last_rows, int n_req,
                    int max_kvlen, const vox_sampling_config* sampling, uint64_t seed, int feedback);
 
+/* ---- hybrid-mixer LM engine ---------------------------------------------------------------------------------
+ * A decoder whose layers mix tokens with a linear recurrence (HGRN2, mLSTM) or with sliding-window attention over a
+ * paged cache that also keeps one mean key / value per block of older tokens; a contiguous range of layers may run
+ * several times with the same weights (every run owns its cache or state).  Residual stream, norms, rotary angles,
+ * scores, gates and recurrent states are fp32 in both dtypes; the dtype is the storage of the matrices and of the
+ * K / V cache and the GEMM operand precision.  One step = a ragged set of rows (prompt portions next to single
+ * decoded tokens); rows of a request are contiguous and ascending in position.                                     */
+typedef struct vox_hybrid vox_hybrid;
+enum { VOX_MIXER_HGRN2 = 0, VOX_MIXER_POOLED_WINDOW_ATTN = 1, VOX_MIXER_MLSTM = 2 };
+enum { VOX_HYBRID_BF16 = 0, VOX_HYBRID_F32 = 1 };
+typedef struct {
+    int32_t kind, heads, kv_heads, dim, vdim;
+    int32_t window, pool, rot_dims;       /* attention: visible tokens, tokens per pooled block, rotated dims per head */
+    float scale, gate_cap;                /* attention score scale; mLSTM soft cap of the gate pre-activations */
+    int32_t ff;                           /* feed-forward width, 0 = the layer has none */
+    const float *norm1, *norm2;           /* [width] fp32 */
+    /* fused input projection, rows in this order:
+     *   HGRN2      q (heads*dim) | forget (heads*dim) | v (heads*vdim)
+     *   attention  q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim) | output gate (heads)
+     *   mLSTM      q (heads*dim) | k (heads*dim) | v (heads*vdim) | output gate (heads*vdim) | input gate (heads) | forget gate (heads) */
+    const void* w_in;                     /* [n_in, width] engine dtype */
+    const float* b_in;                    /* [n_in] fp32 or NULL */
+    const void* w_out;                    /* [width, heads*vdim] */
+    const float* lower;                   /* HGRN2: lower bound of the forget gate [heads*dim] */
+    const float* head_norm;               /* HGRN2: [vdim] shared by heads; mLSTM: [heads*vdim] */
+    const float* inv_freq;                /* attention: rotary frequencies [rot_dims/2] (scaling already applied) */
+    const void *w_up, *w_down;            /* [ff, width], [width, ff] */
+} vox_hybrid_layer;
+typedef struct {
+    int32_t layer;       /* index into layers */
+    int32_t loop_in;     /* 1: x <- loop_in [x; x0] before this run */
+    void* cache;         /* attention: K [max_pages*page_size][kv_heads*dim] then V [max_pages*page_size][kv_heads*vdim], engine dtype */
+    float* pool;         /* attention: [max_pages][(page_size-1)/pool+1][kv_heads][dim+vdim] */
+    float* state;        /* HGRN2: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1] */
+} vox_hybrid_run;
+typedef struct {
+    int32_t width, vocab, n_layers, n_runs, dtype, page_size, max_rows, max_batch, max_out, max_pages;
+    float eps;
+} vox_hybrid_config;
+typedef struct {
+    const vox_hybrid_layer* layers;
+    const vox_hybrid_run* runs;
+    const void *embedding /*[vocab,width]*/, *loop_in /*[width,2*width] or NULL*/, *head /*[vocab,width]*/;
+    const float* final_norm;
+} vox_hybrid_weights;
+typedef struct {
+    const int32_t *pos, *row_req, *page, *slot;   /* per row: position, request index in this step, K/V page and slot */
+    const int32_t* req_rows;                      /* [n_req+1] first row of each request */
+    const int32_t* req_state;                     /* [n_req] recurrent-state slot */
+    const int32_t* page_table;                    /* [n_req][pt_stride] page of token block j */
+    int32_t pt_stride;
+    const int32_t* out_rows;                      /* [n_out] rows whose logits are produced */
+    float* logits;                                /* [n_out, vocab] fp32 */
+    float* trace;                                 /* optional [n_runs][max_rows][width]: residual stream after every run */
+    int32_t *input_ids, *out_ids;                 /* [max_batch] decode inputs (feedback target) and sampled ids */
+    uint64_t* rng_offset;
+} vox_hybrid_io;
+int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybrid_weights* w, vox_hybrid** out);
+void vox_hybrid_destroy(vox_hybrid* m);
+/* ids: [n_rows] token ids of the rows.  sampling NULL: logits only; else one pick per request from output rows 0..n_req-1. */
+int vox_hybrid_step(vox_hybrid* m, void* stream, const vox_hybrid_io* io, const int32_t* ids, int n_rows, int n_req, int n_out,
+                    const vox_sampling_config* sampling, uint64_t seed, int feedback);
+
 /* ---- Qwen3-TTS 12 Hz codec decoder (token -> waveform), streaming ------------------------------------
  * replaces Qwen3TTSTokenizerV2Decoder.forward_chunk (tokenizer/qwen3_codec.py:1541-1666), the DecoderCache
  * plumbing (tokenizer/base.py:7-173) and CudaGraphWorker.run_detokenize's cache cat / copy-in / copy-out

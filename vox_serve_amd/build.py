@@ -6,9 +6,11 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libvoxhip.so")
-SOURCES = ["kernels_lm.hip", "sampler.hip", "engine.hip", "codec.hip"]
+SOURCES = ["kernels_lm.hip", "sampler.hip", "engine.hip", "codec.hip", "hybrid.hip"]
 # -ffp-contract=off: the numeric contract spells every fused multiply-add as an explicit fmaf
-FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC", "-Wno-unused-value"] + \
+# -packed-fp32-ops off: no packed fp32 instructions are generated from scalar float code (same results, instruction by instruction)
+FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-ffp-contract=off", "-fPIC", "-Wno-unused-value",
+         "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"] + \
     os.environ.get("VOX_EXTRA_FLAGS", "").split()
 
 

@@ -1,0 +1,780 @@
+// Hybrid-mixer LM engine: a decoder whose layers mix tokens either with a linear recurrence (HGRN2, mLSTM) or with
+// sliding-window attention over a paged cache that also keeps one mean key / value per block of older tokens.  A contiguous
+// range of layers may run several times with the same weights; every run owns its cache or recurrent state.
+//
+// Numeric rule of this engine: the residual stream, norms, rotary angles, attention scores / softmax, gates, decays and every
+// recurrent state are fp32.  The engine's dtype (bf16 or fp32) is the storage of the large matrices, of the K / V cache and of
+// the GEMM operands (fp32 accumulation either way); fp32 mode multiplies in plain fp32 FMA.
+// One step = a ragged set of rows: each request contributes its next tokens (a prompt portion or one decoded token); rows of
+// one request are contiguous and in position order.  Nothing a row computes depends on which other rows share the step:
+// every reduction runs in an order fixed by the row's own sizes.
+#include <math.h>
+
+#include <vector>
+
+#include "vox_internal.h"
+
+namespace {
+
+typedef __bf16 hb_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float hb_f32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ float hb_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float hb_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float hb_sigmoid(float x) { return 1.0f / (1.0f + expf(-x)); }
+__device__ __forceinline__ float hb_logsigmoid(float x) { return fminf(x, 0.0f) - log1pf(expf(-fabsf(x))); }
+
+__device__ __forceinline__ float hb_ld(const float* p) { return *p; }
+__device__ __forceinline__ float hb_ld(const bf16_t* p) { return bf2f(*p); }
+__device__ __forceinline__ void hb_st(float* p, float v) { *p = v; }
+__device__ __forceinline__ void hb_st(bf16_t* p, float v) { *p = f2bf(v); }
+// what a GEMM operand of the engine's dtype sees of an fp32 activation
+template <typename T> __device__ __forceinline__ float hb_operand(float v);
+template <> __device__ __forceinline__ float hb_operand<float>(float v) { return v; }
+template <> __device__ __forceinline__ float hb_operand<bf16_t>(float v) { return bfround(v); }
+
+enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2 };
+template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float acc, float bias) {
+    float v = acc + bias;
+    if (EPI == HB_EPI_GELU) v = 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    if (EPI == HB_EPI_RESID) v = *c + v;
+    *c = v;
+}
+
+// ---- embedding gather: x[row] = table[id]; the second half of both residual buffers keeps the embedding output ----------
+template <typename T>
+__global__ __launch_bounds__(256) void k_hb_embed(const T* table, const int* ids, int id_stride, float* xa, float* xb, int W, int vocab) {
+    const int row = blockIdx.x;
+    int id = ids[(size_t)row * id_stride];
+    id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float v = hb_ld(table + (size_t)id * W + i);
+        xa[(size_t)row * 2 * W + i] = v;
+        xa[(size_t)row * 2 * W + W + i] = v;
+        xb[(size_t)row * 2 * W + W + i] = v;
+    }
+}
+
+// ---- layer norm with a weight and no bias, fp32; optional row gather ----------------------------------------------------
+__global__ __launch_bounds__(256) void k_hb_layernorm(const float* x, long ldx, const int* rows, const float* w, float* y, long ldy, int W,
+                                                      float eps) {
+    __shared__ float red[4];
+    const int r = blockIdx.x, src = rows ? rows[r] : r;
+    const float* xr = x + (size_t)src * ldx;
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    float s = 0.f;
+    for (int i = threadIdx.x; i < W; i += 256) s += xr[i];
+    s = hb_wave_sum(s);
+    if (lane == 0) red[wv] = s;
+    __syncthreads();
+    const float mean = (((red[0] + red[1]) + red[2]) + red[3]) / (float)W;
+    __syncthreads();
+    float q = 0.f;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float d = xr[i] - mean;
+        q += d * d;
+    }
+    q = hb_wave_sum(q);
+    if (lane == 0) red[wv] = q;
+    __syncthreads();
+    const float var = (((red[0] + red[1]) + red[2]) + red[3]) / (float)W;
+    const float inv = 1.0f / sqrtf(var + eps);
+    for (int i = threadIdx.x; i < W; i += 256) y[(size_t)r * ldy + i] = (xr[i] - mean) * inv * w[i];
+}
+
+// ---- GEMM  C[M,N] (+)= A[M,K] . W[N,K]^T + bias ---------------------------------------------------------------------------
+// bf16: both operands staged in LDS as bf16 (activations rounded once), v_mfma_f32_16x16x32_bf16; four waves, 64 output columns
+// per block, BM = 64 (2 x 2 tiles per wave) or BM = 16 (one tile per wave).  Every edge (M, N, K) is guarded at the LDS fill.
+template <int BM, int EPI>
+__global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, const bf16_t* Wt, const float* bias, float* C, long ldc, int M,
+                                                      int N, int K) {
+    constexpr int BK = 64, LD = BK + 8;
+    __shared__ __attribute__((aligned(16))) bf16_t As[BM * LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Ws[64 * LD];
+    const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
+    constexpr int MT = BM == 64 ? 2 : 1, NT = BM == 64 ? 2 : 1;
+    const int mt0 = BM == 64 ? (wv >> 1) * 2 : 0, nt0 = BM == 64 ? (wv & 1) * 2 : wv;
+    hb_f32x4 acc[MT][NT];
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) acc[i][j] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
+    const bool a_vec = (K % 4 == 0) && (lda % 4 == 0) && ((((size_t)A) & 15) == 0);
+    const bool w_vec = (K % 8 == 0) && ((((size_t)Wt) & 15) == 0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        // A tile: BM x 64 fp32 -> bf16
+        for (int idx = tid; idx < BM * 16; idx += 256) {
+            const int r = idx >> 4, c = (idx & 15) * 4;
+            const int gm = m0 + r, gk = k0 + c;
+            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+            if (gm < M) {
+                const float* p = A + (size_t)gm * lda + gk;
+                if (a_vec && gk + 3 < K) v = *(const float4*)p;
+                else {
+                    if (gk < K) v.x = p[0];
+                    if (gk + 1 < K) v.y = p[1];
+                    if (gk + 2 < K) v.z = p[2];
+                    if (gk + 3 < K) v.w = p[3];
+                }
+            }
+            uint2 o;
+            o.x = pack_bf2(v.x, v.y);
+            o.y = pack_bf2(v.z, v.w);
+            *(uint2*)(As + r * LD + c) = o;
+        }
+        // W tile: 64 x 64 bf16
+        for (int idx = tid; idx < 64 * 8; idx += 256) {
+            const int r = idx >> 3, c = (idx & 7) * 8;
+            const int gn = n0 + r, gk = k0 + c;
+            uint4 v = make_uint4(0, 0, 0, 0);
+            if (gn < N) {
+                const bf16_t* p = Wt + (size_t)gn * K + gk;
+                if (w_vec && gk + 7 < K) v = *(const uint4*)p;
+                else {
+                    bf16_t t[8];
+#pragma unroll
+                    for (int e = 0; e < 8; ++e) t[e] = gk + e < K ? p[e] : (bf16_t)0;
+                    v.x = t[0] | ((u32)t[1] << 16); v.y = t[2] | ((u32)t[3] << 16);
+                    v.z = t[4] | ((u32)t[5] << 16); v.w = t[6] | ((u32)t[7] << 16);
+                }
+            }
+            *(uint4*)(Ws + r * LD + c) = v;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int ks = 0; ks < BK; ks += 32) {
+            hb_bf16x8 af[MT], bfr[NT];
+#pragma unroll
+            for (int i = 0; i < MT; ++i) {
+                union { uint4 u; hb_bf16x8 b; } cv;
+                cv.u = *(const uint4*)(As + ((mt0 + i) * 16 + (lane & 15)) * LD + ks + (lane >> 4) * 8);
+                af[i] = cv.b;
+            }
+#pragma unroll
+            for (int j = 0; j < NT; ++j) {
+                union { uint4 u; hb_bf16x8 b; } cv;
+                cv.u = *(const uint4*)(Ws + ((nt0 + j) * 16 + (lane & 15)) * LD + ks + (lane >> 4) * 8);
+                bfr[j] = cv.b;
+            }
+#pragma unroll
+            for (int i = 0; i < MT; ++i)
+#pragma unroll
+                for (int j = 0; j < NT; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < MT; ++i)
+#pragma unroll
+        for (int j = 0; j < NT; ++j) {
+            const int gn = n0 + (nt0 + j) * 16 + (lane & 15);
+            if (gn >= N) continue;
+            const float b = bias ? bias[gn] : 0.f;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int gm = m0 + (mt0 + i) * 16 + (lane >> 4) * 4 + r;
+                if (gm < M) hb_epilogue<EPI>(C + (size_t)gm * ldc + gn, acc[i][j][r], b);
+            }
+        }
+}
+
+// fp32: LDS-tiled FMA, 64 output columns per block, BM = 64 (4 x 4 per thread) or 16 (1 x 4 per thread); k ascending per element.
+template <int BM, int EPI>
+__global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, const float* Wt, const float* bias, float* C, long ldc, int M,
+                                                     int N, int K) {
+    constexpr int BK = 16, RM = BM / 16;
+    __shared__ float As[BK][BM + 4];
+    __shared__ float Ws[BK][64 + 4];
+    const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
+    const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
+    float acc[RM][4];
+#pragma unroll
+    for (int i = 0; i < RM; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+    for (int k0 = 0; k0 < K; k0 += BK) {
+        for (int idx = tid; idx < BM * BK; idx += 256) {
+            const int r = idx / BK, c = idx % BK;
+            const int gm = m0 + r, gk = k0 + c;
+            As[c][r] = (gm < M && gk < K) ? A[(size_t)gm * lda + gk] : 0.f;
+        }
+        for (int idx = tid; idx < 64 * BK; idx += 256) {
+            const int r = idx / BK, c = idx % BK;
+            const int gn = n0 + r, gk = k0 + c;
+            Ws[c][r] = (gn < N && gk < K) ? Wt[(size_t)gn * K + gk] : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BK; ++k) {
+            float a[RM], b[4];
+#pragma unroll
+            for (int i = 0; i < RM; ++i) a[i] = As[k][ty * RM + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = Ws[k][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < RM; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < RM; ++i) {
+        const int gm = m0 + ty * RM + i;
+        if (gm >= M) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int gn = n0 + tx * 4 + j;
+            if (gn < N) hb_epilogue<EPI>(C + (size_t)gm * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f);
+        }
+    }
+}
+
+// 1..8 rows (decode): one wave per output column streams its weight row once, 16 bytes per lane and request; lanes own
+// k-chunks c, c + 64, ...; butterfly at the end.
+template <typename T, int MR, int EPI>
+__global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const T* Wt, const float* bias, float* C, long ldc, int M, int N,
+                                                 int K) {
+    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+    const T* wr = Wt + (size_t)n * K;
+    const bool vec = (K % CH == 0) && ((((size_t)Wt) & 15) == 0) && (lda % 4 == 0) && ((((size_t)A) & 15) == 0);
+    if (vec) {
+        for (int k = lane * CH; k < K; k += 64 * CH) {
+            float w[CH];
+            if (sizeof(T) == 2) {
+                const uint4 u = *(const uint4*)(wr + k);
+                w[0] = bflo(u.x); w[1] = bfhi(u.x); w[2] = bflo(u.y); w[3] = bfhi(u.y);
+                if (CH == 8) { w[4] = bflo(u.z); w[5] = bfhi(u.z); w[6] = bflo(u.w); w[7] = bfhi(u.w); }
+            } else {
+                const float4 u = *(const float4*)(wr + k);
+                w[0] = u.x; w[1] = u.y; w[2] = u.z; w[3] = u.w;
+            }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                if (m >= M) break;
+                const float* xr = A + (size_t)m * lda + k;
+#pragma unroll
+                for (int e = 0; e < CH; e += 4) {
+                    const float4 x = *(const float4*)(xr + e);
+                    acc[m] = fmaf(w[e], hb_operand<T>(x.x), acc[m]);
+                    acc[m] = fmaf(w[e + 1], hb_operand<T>(x.y), acc[m]);
+                    acc[m] = fmaf(w[e + 2], hb_operand<T>(x.z), acc[m]);
+                    acc[m] = fmaf(w[e + 3], hb_operand<T>(x.w), acc[m]);
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) {
+            const float w = hb_ld(wr + k);
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+                if (m < M) acc[m] = fmaf(w, hb_operand<T>(A[(size_t)m * lda + k]), acc[m]);
+        }
+    }
+    const float b = bias ? bias[n] : 0.f;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        const float s = hb_wave_sum(acc[m]);
+        if (m < M && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n, s, b);
+    }
+}
+
+template <typename T, int EPI>
+int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K);
+
+template <int EPI>
+int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K) {
+    if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_bf16<16, EPI>), dim3((N + 63) / 64, 1), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    else hipLaunchKernelGGL((k_hb_gemm_bf16<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    return VOX_OK;
+}
+template <int EPI>
+int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const float* W, const float* bias, float* C, long ldc, int M, int N, int K) {
+    if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_f32<16, EPI>), dim3((N + 63) / 64, 1), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    else hipLaunchKernelGGL((k_hb_gemm_f32<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    return VOX_OK;
+}
+template <typename T, int EPI>
+int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
+    if (M <= 0 || N <= 0) return VOX_OK;
+    const dim3 g((N + 3) / 4), b(256);
+    if (M == 1) hipLaunchKernelGGL((k_hb_gemv<T, 1, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    else if (M == 2) hipLaunchKernelGGL((k_hb_gemv<T, 2, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    else if (M <= 4) hipLaunchKernelGGL((k_hb_gemv<T, 4, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    else if (M <= 8) hipLaunchKernelGGL((k_hb_gemv<T, 8, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    else return hb_gemm_tiles<EPI>(st, A, lda, W, bias, C, ldc, M, N, K);
+    return VOX_OK;
+}
+template <typename T>
+int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
+    if (epi == HB_EPI_GELU) return hb_gemm_epi<T, HB_EPI_GELU>(st, A, lda, W, bias, C, ldc, M, N, K);
+    if (epi == HB_EPI_RESID) return hb_gemm_epi<T, HB_EPI_RESID>(st, A, lda, W, bias, C, ldc, M, N, K);
+    return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K);
+}
+
+// ---- HGRN2: S_t = diag(f_t) S_{t-1} + (1 - f_t) v_t^T,  o_t = S_t^T q_t ---------------------------------------------------
+// proj row = [q (H*dim) | f (H*dim) | v (H*vdim)] pre-activation (bias already added).  One wave per (request, head, 64 value
+// columns): the state tile lives in LDS for the whole portion and goes back to its slot at the end.
+__global__ __launch_bounds__(64) void k_hb_hgrn2_scan(const float* proj, long ldp, float* out, long ldo, const float* lower, float* state,
+                                                      const int* req_rows, const int* req_state, const int* pos, int H, int dim, int vdim) {
+    extern __shared__ float sm[];
+    float* S = sm;                 // [dim][64]
+    float* fs = sm + dim * 64;     // [dim]
+    float* qs = fs + dim;          // [dim]
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, c = blockIdx.z * 64 + lane;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const bool ok = c < vdim, fresh = pos[rs] == 0;
+    float* St = state + ((size_t)req_state[r] * H + h) * dim * vdim;
+    for (int d = 0; d < dim; ++d) S[d * 64 + lane] = (ok && !fresh) ? St[(size_t)d * vdim + c] : 0.f;
+    for (int t = rs; t < re; ++t) {
+        const float* p = proj + (size_t)t * ldp;
+        for (int d = lane; d < dim; d += 64) {
+            const float qv = p[h * dim + d];
+            qs[d] = qv * hb_sigmoid(qv);
+            const float lo = lower[h * dim + d];
+            fs[d] = lo + (1.0f - lo) * hb_sigmoid(p[H * dim + h * dim + d]);
+        }
+        __syncthreads();
+        const float v = ok ? p[2 * H * dim + h * vdim + c] : 0.f;
+        float o = 0.f;
+        for (int d = 0; d < dim; ++d) {
+            const float f = fs[d];
+            const float s = f * S[d * 64 + lane] + (1.0f - f) * v;
+            S[d * 64 + lane] = s;
+            o = fmaf(s, qs[d], o);
+        }
+        if (ok) out[(size_t)t * ldo + h * vdim + c] = o;
+        __syncthreads();
+    }
+    if (ok)
+        for (int d = 0; d < dim; ++d) St[(size_t)d * vdim + c] = S[d * 64 + lane];
+}
+
+// ---- mLSTM with the running-maximum stabiliser -------------------------------------------------------------------------------
+// proj row = [q (H*dim) | k (H*dim) | v (H*vdim) | g (H*vdim) | i (H) | f (H)].  State per (slot, head): S [dim][vdim], n [dim], m.
+// Every value tile keeps its own copy of n and m (same arithmetic, same order); tile 0 writes them back.
+__global__ __launch_bounds__(64) void k_hb_mlstm_scan(const float* proj, long ldp, float* out, long ldo, float* state, const int* req_rows,
+                                                      const int* req_state, const int* pos, int H, int dim, int vdim, float cap) {
+    extern __shared__ float sm[];
+    float* S = sm;                 // [dim][64]
+    float* ns = sm + dim * 64;     // [dim]
+    float* ks = ns + dim;          // [dim]
+    float* qs = ks + dim;          // [dim]
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, c = blockIdx.z * 64 + lane;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const bool ok = c < vdim, fresh = pos[rs] == 0;
+    const size_t per = (size_t)dim * vdim + dim + 1;
+    float* St = state + ((size_t)req_state[r] * H + h) * per;
+    float* nt = St + (size_t)dim * vdim;
+    for (int d = 0; d < dim; ++d) S[d * 64 + lane] = (ok && !fresh) ? St[(size_t)d * vdim + c] : 0.f;
+    for (int d = lane; d < dim; d += 64) ns[d] = fresh ? 0.f : nt[d];
+    float m = fresh ? 0.f : nt[dim];
+    const float qscale = 1.0f / sqrtf((float)dim);
+    const int off_k = H * dim, off_v = 2 * H * dim, off_i = 2 * H * dim + 2 * H * vdim, off_f = off_i + H;
+    __syncthreads();
+    for (int t = rs; t < re; ++t) {
+        const float* p = proj + (size_t)t * ldp;
+        const float ig = cap * tanhf(p[off_i + h] / cap);
+        const float fg = hb_logsigmoid(cap * tanhf(p[off_f + h] / cap));
+        const float mn = fmaxf(fg + m, ig);
+        const float a = expf(fg + m - mn), b = expf(ig - mn);
+        float part = 0.f;
+        for (int d = lane; d < dim; d += 64) {
+            const float kv = p[off_k + h * dim + d], qv = p[h * dim + d] * qscale;
+            const float nn = a * ns[d] + b * kv;
+            ns[d] = nn;
+            ks[d] = kv;
+            qs[d] = qv;
+            part = fmaf(nn, qv, part);
+        }
+        const float nq = hb_wave_sum(part);
+        __syncthreads();
+        const float v = ok ? p[off_v + h * vdim + c] : 0.f;
+        const float bv = b * v;
+        float o = 0.f;
+        for (int d = 0; d < dim; ++d) {
+            const float s = a * S[d * 64 + lane] + ks[d] * bv;
+            S[d * 64 + lane] = s;
+            o = fmaf(s, qs[d], o);
+        }
+        m = mn;
+        const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
+        if (ok) out[(size_t)t * ldo + h * vdim + c] = o / den;
+        __syncthreads();
+    }
+    if (ok)
+        for (int d = 0; d < dim; ++d) St[(size_t)d * vdim + c] = S[d * 64 + lane];
+    if (blockIdx.z == 0) {
+        for (int d = lane; d < dim; d += 64) nt[d] = ns[d];
+        if (lane == 0) nt[dim] = m;
+    }
+}
+
+// per (row, head): o / rms(o) over vdim, times a weight (per_head_w: indexed over all heads, else shared [vdim]), times
+// sigmoid(gate) when gate_off >= 0 (gate = proj[row][gate_off + h*vdim + j]).  In place.
+__global__ __launch_bounds__(64) void k_hb_head_norm(float* o, long ldo, const float* w, int per_head_w, const float* proj, long ldp, int gate_off,
+                                                     int vdim, float eps) {
+    const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
+    float* p = o + (size_t)row * ldo + (size_t)h * vdim;
+    float ss = 0.f;
+    for (int j = lane; j < vdim; j += 64) ss = fmaf(p[j], p[j], ss);
+    ss = hb_wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
+    for (int j = lane; j < vdim; j += 64) {
+        float v = p[j] * inv * w[per_head_w ? h * vdim + j : j];
+        if (gate_off >= 0) v *= hb_sigmoid(proj[(size_t)row * ldp + gate_off + h * vdim + j]);
+        p[j] = v;
+    }
+}
+
+// ---- attention: rotary (interleaved pairs, first `rot` dims) + unit RMS on q and k, K / V into the paged cache -----------
+// proj row = [q (H*dim) | k (G*dim) | v (G*vdim) | gate (H)].  Cache of one run: K [pages*ps][G*dim] then V [pages*ps][G*vdim].
+#define HB_MAX_DPL 8   // dims per lane: dim <= 512
+template <typename T>
+__global__ __launch_bounds__(64) void k_hb_attn_prep(float* proj, long ldp, T* cache, const float* inv_freq, const int* pos, const int* page,
+                                                     const int* slot, int H, int G, int dim, int vdim, int rot, int ps, long v_base, float eps) {
+    const int row = blockIdx.x, hb = blockIdx.y, lane = threadIdx.x;
+    const bool is_q = hb < H;
+    const int g = hb - H;
+    float* src = proj + (size_t)row * ldp + (is_q ? hb * dim : H * dim + g * dim);
+    const float p = (float)pos[row];
+    float y[HB_MAX_DPL];
+    float ss = 0.f;
+#pragma unroll
+    for (int e = 0; e < HB_MAX_DPL; ++e) {
+        const int d = lane + e * 64;
+        y[e] = 0.f;
+        if (d < dim) {
+            float v = src[d];
+            if (d < rot) {
+                const float ang = p * inv_freq[d >> 1];
+                float sn, cs;
+                sincosf(ang, &sn, &cs);
+                const float other = src[d ^ 1];
+                v = (d & 1) ? (v * cs + other * sn) : (v * cs - other * sn);
+            }
+            y[e] = v;
+            ss = fmaf(v, v, ss);
+        }
+    }
+    ss = hb_wave_sum(ss);
+    const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+    const size_t tok = (size_t)page[row] * ps + slot[row];
+    // every lane has read its inputs (both pair members) before anyone overwrites: one wave, the reduction above is the fence
+#pragma unroll
+    for (int e = 0; e < HB_MAX_DPL; ++e) {
+        const int d = lane + e * 64;
+        if (d < dim) {
+            if (is_q) src[d] = y[e] * inv;
+            else hb_st(cache + tok * (size_t)(G * dim) + g * dim + d, y[e] * inv);
+        }
+    }
+    if (!is_q) {
+        const float* vs = proj + (size_t)row * ldp + H * dim + G * dim + g * vdim;
+        for (int j = lane; j < vdim; j += 64) hb_st(cache + v_base + tok * (size_t)(G * vdim) + g * vdim + j, vs[j]);
+    }
+}
+
+// mean key / value of a block of `P` tokens, taken from the cache as stored, when the row's token closes the block.
+// pool entry of block b sits with the page of the block's last token t: pool[(page(t) * ppp + (t % ps) / P)][G][dim + vdim].
+template <typename T>
+__global__ __launch_bounds__(64) void k_hb_pool_update(const T* cache, float* pool, const int* pos, const int* row_req, const int* ptab,
+                                                       int pts, int G, int dim, int vdim, int P, int ps, int ppp, long v_base) {
+    const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x;
+    const int p = pos[row];
+    if ((p + 1) % P != 0) return;
+    const int* pt = ptab + (size_t)row_req[row] * pts;
+    const size_t entry = (size_t)pt[p / ps] * ppp + (p % ps) / P;
+    float* dst = pool + (entry * G + g) * (size_t)(dim + vdim);
+    for (int d = lane; d < dim + vdim; d += 64) {
+        float s = 0.f;
+        for (int j = p - P + 1; j <= p; ++j) {
+            const size_t tok = (size_t)pt[j / ps] * ps + j % ps;
+            s += d < dim ? hb_ld(cache + tok * (size_t)(G * dim) + g * dim + d)
+                         : hb_ld(cache + v_base + tok * (size_t)(G * vdim) + g * vdim + (d - dim));
+        }
+        dst[d] = s / (float)P;
+    }
+}
+
+// One block per (row, kv head); one wave per query head of the group.  Keys of a row at position p: the pooled blocks
+// 0 .. nb-1 (nb = floor((p - window + 1) / P), those wholly before the window) and then the tokens max(0, p-window+1) .. p.
+// 64 keys at a time: lane = key (score), then lane = value column; running maximum / sum across the chunks in ascending order.
+#define HB_MAX_VPL 8   // value columns per lane: vdim <= 512
+template <typename T>
+__global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
+                          const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
+                          long v_base, float scale) {
+    extern __shared__ float sm[];
+    const int QG = H / G;
+    long* loc = (long*)sm;                 // [QG][64]  (>= 0: token index in the cache, < 0: -(pool entry) - 1)
+    float* pr = sm + QG * 128;             // [QG][64]
+    float* qs = pr + QG * 64;              // [QG][dim]
+    const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int hq = g * QG + wv;
+    const int p = pos[row];
+    const int* pt = ptab + (size_t)row_req[row] * pts;
+    const int first = p - window + 1;
+    const int lo = first > 0 ? first : 0;
+    const int nb = first > 0 ? first / P : 0;
+    const int total = nb + (p - lo + 1);
+    const float* q = proj + (size_t)row * ldp + hq * dim;
+    for (int d = lane; d < dim; d += 64) qs[wv * dim + d] = q[d];
+    __syncthreads();
+    float m = -INFINITY, l = 0.f, acc[HB_MAX_VPL];
+#pragma unroll
+    for (int e = 0; e < HB_MAX_VPL; ++e) acc[e] = 0.f;
+    const int pw = dim + vdim;
+    for (int base = 0; base < total; base += 64) {
+        const int u = base + lane;
+        float s = -INFINITY;
+        long where = 0;
+        if (u < total) {
+            float dot = 0.f;
+            if (u < nb) {
+                const int t = u * P + P - 1;
+                const size_t entry = ((size_t)pt[t / ps] * ppp + (t % ps) / P) * G + g;
+                const float* kp = pool + entry * pw;
+                for (int d = 0; d < dim; ++d) dot = fmaf(qs[wv * dim + d], kp[d], dot);
+                where = -(long)entry - 1;
+            } else {
+                const int j = lo + (u - nb);
+                const size_t tok = (size_t)pt[j / ps] * ps + j % ps;
+                const T* kp = cache + tok * (size_t)(G * dim) + g * dim;
+                for (int d = 0; d < dim; ++d) dot = fmaf(qs[wv * dim + d], hb_ld(kp + d), dot);
+                where = (long)tok;
+            }
+            s = dot * scale;
+        }
+        const float mn = fmaxf(m, hb_wave_max(s));
+        const float alpha = expf(m - mn);
+        const float e = u < total ? expf(s - mn) : 0.f;
+        l = l * alpha + hb_wave_sum(e);
+        m = mn;
+        pr[wv * 64 + lane] = e;
+        loc[wv * 64 + lane] = where;
+        __syncthreads();
+        const int cnt = total - base < 64 ? total - base : 64;
+#pragma unroll
+        for (int c = 0; c < HB_MAX_VPL; ++c) {
+            const int j = lane + c * 64;
+            if (j < vdim) {
+                float a = acc[c] * alpha;
+                for (int kk = 0; kk < cnt; ++kk) {
+                    const long w = loc[wv * 64 + kk];
+                    const float vv = w < 0 ? pool[(size_t)(-w - 1) * pw + dim + j]
+                                           : hb_ld(cache + v_base + (size_t)w * (size_t)(G * vdim) + g * vdim + j);
+                    a = fmaf(pr[wv * 64 + kk], vv, a);
+                }
+                acc[c] = a;
+            }
+        }
+        __syncthreads();
+    }
+    const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
+#pragma unroll
+    for (int c = 0; c < HB_MAX_VPL; ++c) {
+        const int j = lane + c * 64;
+        if (j < vdim) out[(size_t)row * ldo + hq * vdim + j] = acc[c] / l * gate;
+    }
+}
+
+__global__ void k_hb_copy_rows(const float* src, long lds_, float* dst, long ldd, int W) {
+    const int row = blockIdx.x;
+    for (int i = threadIdx.x; i < W; i += blockDim.x) dst[(size_t)row * ldd + i] = src[(size_t)row * lds_ + i];
+}
+__global__ void k_hb_logits_bf16(const float* src, bf16_t* dst, long n) {
+    const long i = (long)blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = f2bf(src[i]);
+}
+__global__ void k_hb_feedback(const int* out_ids, int* input_ids, uint64_t* rng, int B, int feedback) {
+    const int b = blockIdx.x * blockDim.x + threadIdx.x;
+    if (feedback && b < B) input_ids[b] = out_ids[b];
+    if (b == 0 && rng) *rng += 1;
+}
+
+}  // namespace
+
+struct vox_hybrid {
+    vox_ctx* ctx;
+    vox_hybrid_config cfg;
+    std::vector<vox_hybrid_layer> layers;
+    std::vector<vox_hybrid_run> runs;
+    vox_hybrid_weights w;
+    float *xa = nullptr, *xb = nullptr, *h = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
+    bf16_t* logits16 = nullptr;
+    int max_in = 0, max_mix = 0, max_ff = 0;
+};
+
+static int hb_layer_in(const vox_hybrid_layer& L) {
+    switch (L.kind) {
+        case VOX_MIXER_HGRN2: return 2 * L.heads * L.dim + L.heads * L.vdim;
+        case VOX_MIXER_POOLED_WINDOW_ATTN: return L.heads * L.dim + L.kv_heads * (L.dim + L.vdim) + L.heads;
+        case VOX_MIXER_MLSTM: return 2 * L.heads * L.dim + 2 * L.heads * L.vdim + 2 * L.heads;
+    }
+    return -1;
+}
+
+template <typename T>
+static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const int32_t* ids, int n, int n_req, int n_out) {
+    const vox_hybrid_config& c = m->cfg;
+    const int W = c.width, ps = c.page_size;
+    const long ldx = 2L * W;
+    hipLaunchKernelGGL((k_hb_embed<T>), dim3(n), dim3(256), 0, st, (const T*)m->w.embedding, ids, 1, m->xa, m->xb, W, c.vocab);
+    float *cur = m->xa, *other = m->xb;
+    for (int ri = 0; ri < c.n_runs; ++ri) {
+        const vox_hybrid_run& run = m->runs[ri];
+        const vox_hybrid_layer& L = m->layers[run.layer];
+        if (run.loop_in) {
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, cur, ldx, (const T*)m->w.loop_in, nullptr, other, ldx, n, W, 2 * W));
+            float* t = cur; cur = other; other = t;
+        }
+        const int n_in = hb_layer_in(L), n_mix = L.heads * L.vdim;
+        hipLaunchKernelGGL(k_hb_layernorm, dim3(n), dim3(256), 0, st, cur, ldx, (const int*)nullptr, L.norm1, m->h, (long)W, W, c.eps);
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->h, W, (const T*)L.w_in, L.b_in, m->proj, n_in, n, n_in, W));
+        const int vt = (L.vdim + 63) / 64;
+        if (L.kind == VOX_MIXER_HGRN2) {
+            const size_t lds = (size_t)(L.dim * 64 + 2 * L.dim) * 4;
+            hipLaunchKernelGGL(k_hb_hgrn2_scan, dim3(n_req, L.heads, vt), dim3(64), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, L.lower,
+                               run.state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim);
+            hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 0, m->proj, (long)n_in, -1,
+                               L.vdim, c.eps);
+        } else if (L.kind == VOX_MIXER_MLSTM) {
+            const size_t lds = (size_t)(L.dim * 64 + 3 * L.dim) * 4;
+            hipLaunchKernelGGL(k_hb_mlstm_scan, dim3(n_req, L.heads, vt), dim3(64), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, run.state,
+                               io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap);
+            hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_in,
+                               2 * L.heads * L.dim + L.heads * L.vdim, L.vdim, c.eps);
+        } else {
+            const int H = L.heads, G = L.kv_heads, QG = H / G;
+            const long v_base = (long)c.max_pages * ps * G * L.dim;
+            const int ppp = (ps - 1) / L.pool + 1;
+            hipLaunchKernelGGL((k_hb_attn_prep<T>), dim3(n, H + G), dim3(64), 0, st, m->proj, (long)n_in, (T*)run.cache, L.inv_freq, io->pos,
+                               io->page, io->slot, H, G, L.dim, L.vdim, L.rot_dims, ps, v_base, c.eps);
+            hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)run.cache, run.pool, io->pos, io->row_req,
+                               io->page_table, io->pt_stride, G, L.dim, L.vdim, L.pool, ps, ppp, v_base);
+            const size_t lds = (size_t)QG * L.dim * 4 + (size_t)QG * 64 * 4 + (size_t)QG * 64 * 8;
+            hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G), dim3(64 * QG), lds, st, m->proj, (long)n_in, (const T*)run.cache, run.pool, m->mix,
+                               (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, L.window, L.pool, ps, ppp,
+                               v_base, L.scale);
+        }
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix));
+        if (L.ff > 0) {
+            hipLaunchKernelGGL(k_hb_layernorm, dim3(n), dim3(256), 0, st, cur, ldx, (const int*)nullptr, L.norm2, m->h, (long)W, W, c.eps);
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff, L.ff, (const T*)L.w_down, nullptr, cur, ldx, n, W, L.ff));
+        }
+        if (io->trace)
+            hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
+    }
+    if (n_out > 0) {
+        hipLaunchKernelGGL(k_hb_layernorm, dim3(n_out), dim3(256), 0, st, cur, ldx, io->out_rows, m->w.final_norm, m->hout, (long)W, W, c.eps);
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits, c.vocab, n_out, c.vocab, W));
+    }
+    VOX_HIP(hipGetLastError());
+    return VOX_OK;
+}
+
+extern "C" {
+
+int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybrid_weights* w, vox_hybrid** out) {
+    if (!ctx || !cfg || !w || !out || !w->layers || !w->runs) return vox_fail(VOX_ERR_INVALID, "hybrid_create: NULL argument");
+    if (cfg->dtype != VOX_HYBRID_BF16 && cfg->dtype != VOX_HYBRID_F32) return vox_fail(VOX_ERR_INVALID, "hybrid_create: dtype %d", cfg->dtype);
+    if (cfg->width < 1 || cfg->vocab < 1 || cfg->page_size < 1 || cfg->max_rows < 1 || cfg->max_batch < 1 || cfg->max_out < 1)
+        return vox_fail(VOX_ERR_INVALID, "hybrid_create: bad sizes");
+    vox_hybrid* m = new vox_hybrid();
+    m->ctx = ctx; m->cfg = *cfg; m->w = *w;
+    m->layers.assign(w->layers, w->layers + cfg->n_layers);
+    m->runs.assign(w->runs, w->runs + cfg->n_runs);
+    m->w.layers = nullptr; m->w.runs = nullptr;
+    for (const vox_hybrid_layer& L : m->layers) {
+        const int n_in = hb_layer_in(L);
+        const char* bad = nullptr;
+        if (n_in < 0) bad = "unknown mixer kind";
+        else if (L.heads < 1 || L.dim < 1 || L.vdim < 1) bad = "heads / dim / vdim";
+        else if (L.vdim > 64 * HB_MAX_VPL) bad = "vdim above 512";
+        else if (!L.norm1 || !L.w_in || !L.w_out) bad = "missing weights";
+        else if (L.ff > 0 && (!L.norm2 || !L.w_up || !L.w_down)) bad = "missing feed-forward weights";
+        else if (L.kind == VOX_MIXER_HGRN2 && (!L.lower || !L.head_norm)) bad = "hgrn2 needs lower and head_norm";
+        else if (L.kind == VOX_MIXER_MLSTM && (!L.head_norm || !(L.gate_cap > 0.f))) bad = "mlstm needs head_norm and gate_cap";
+        else if (L.kind != VOX_MIXER_POOLED_WINDOW_ATTN && (size_t)(L.dim * 64 + 3 * L.dim) * 4 > 160 * 1024) bad = "dim too large for the LDS state tile";
+        else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN) {
+            if (L.kv_heads < 1 || L.heads % L.kv_heads != 0 || L.heads / L.kv_heads > 16) bad = "heads / kv_heads (group of at most 16)";
+            else if (L.dim > 64 * HB_MAX_DPL) bad = "dim above 512";
+            else if (L.window < 1 || L.pool < 1) bad = "window / pool";
+            else if (L.rot_dims < 0 || L.rot_dims > L.dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq)) bad = "rot_dims";
+        }
+        if (bad) { delete m; return vox_fail(VOX_ERR_INVALID, "hybrid_create: layer: %s", bad); }
+        if (n_in > m->max_in) m->max_in = n_in;
+        if (L.heads * L.vdim > m->max_mix) m->max_mix = L.heads * L.vdim;
+        if (L.ff > m->max_ff) m->max_ff = L.ff;
+    }
+    for (const vox_hybrid_run& r : m->runs) {
+        const char* bad = nullptr;
+        if (r.layer < 0 || r.layer >= cfg->n_layers) bad = "layer index";
+        else if (m->layers[r.layer].kind == VOX_MIXER_POOLED_WINDOW_ATTN ? (!r.cache || !r.pool) : !r.state) bad = "missing cache / state";
+        else if (r.loop_in && !w->loop_in) bad = "loop_in weight";
+        if (bad) { delete m; return vox_fail(VOX_ERR_INVALID, "hybrid_create: run: %s", bad); }
+    }
+    const size_t R = cfg->max_rows, W = cfg->width;
+    bool ok = hipMalloc((void**)&m->xa, R * 2 * W * 4) == hipSuccess && hipMalloc((void**)&m->xb, R * 2 * W * 4) == hipSuccess &&
+              hipMalloc((void**)&m->h, R * W * 4) == hipSuccess && hipMalloc((void**)&m->proj, R * (size_t)m->max_in * 4) == hipSuccess &&
+              hipMalloc((void**)&m->mix, R * (size_t)m->max_mix * 4) == hipSuccess &&
+              hipMalloc((void**)&m->ff, R * (size_t)(m->max_ff > 0 ? m->max_ff : 1) * 4) == hipSuccess &&
+              hipMalloc((void**)&m->hout, (size_t)cfg->max_out * W * 4) == hipSuccess &&
+              hipMalloc((void**)&m->logits16, (size_t)cfg->max_batch * cfg->vocab * 2) == hipSuccess;
+    if (!ok) { vox_hybrid_destroy(m); return vox_fail(VOX_ERR_NOMEM, "hybrid_create: hipMalloc failed"); }
+    *out = m;
+    return VOX_OK;
+}
+
+void vox_hybrid_destroy(vox_hybrid* m) {
+    if (!m) return;
+    (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->proj); (void)hipFree(m->mix);
+    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16);
+    delete m;
+}
+
+int vox_hybrid_step(vox_hybrid* m, void* stream, const vox_hybrid_io* io, const int32_t* ids, int n_rows, int n_req, int n_out,
+                    const vox_sampling_config* sc, uint64_t seed, int feedback) {
+    if (!m || !io || !ids) return vox_fail(VOX_ERR_INVALID, "hybrid_step: NULL");
+    const vox_hybrid_config& c = m->cfg;
+    if (n_rows < 1 || n_rows > c.max_rows || n_req < 1 || n_req > c.max_batch || n_req > n_rows || n_out < 0 || n_out > c.max_out)
+        return vox_fail(VOX_ERR_INVALID, "hybrid_step: rows %d / requests %d / outputs %d out of range", n_rows, n_req, n_out);
+    if (!io->pos || !io->row_req || !io->page || !io->slot || !io->req_rows || !io->req_state || !io->page_table || (n_out && (!io->out_rows || !io->logits)))
+        return vox_fail(VOX_ERR_INVALID, "hybrid_step: missing plan arrays");
+    hipStream_t st = (hipStream_t)stream;
+    VOX_TRY(c.dtype == VOX_HYBRID_F32 ? hb_step<float>(m, st, io, ids, n_rows, n_req, n_out) : hb_step<bf16_t>(m, st, io, ids, n_rows, n_req, n_out));
+    if (!sc) return VOX_OK;
+    // sampling: one pick per request from the first n_req output rows (the caller lists each request's last row first)
+    if (n_out < n_req || n_req > c.max_batch || !io->out_ids) return vox_fail(VOX_ERR_INVALID, "hybrid_step: sampling needs one output row per request");
+    const long nl = (long)n_req * c.vocab;
+    hipLaunchKernelGGL(k_hb_logits_bf16, dim3((unsigned)((nl + 255) / 256)), dim3(256), 0, st, io->logits, m->logits16, nl);
+    SampleCall s;
+    s.logits = m->logits16; s.B = n_req; s.V = c.vocab; s.cfg = *sc; s.cfg.repetition_penalty = 1.0f; s.seed = seed; s.offset = 0;
+    s.offset_dev = io->rng_offset; s.offset_mul = 1; s.out_ids = io->out_ids; s.out_stride = 1; s.out_col = 0;
+    s.ws = m->ctx->samp_ws;
+    VOX_TRY(vox_launch_sample(st, s));
+    if (feedback || io->rng_offset)
+        hipLaunchKernelGGL(k_hb_feedback, dim3((n_req + 63) / 64), dim3(64), 0, st, io->out_ids, io->input_ids, io->rng_offset, n_req,
+                           feedback && io->input_ids ? 1 : 0);
+    return VOX_OK;
+}
+
+}  // extern "C"

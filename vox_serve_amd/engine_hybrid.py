@@ -1,0 +1,245 @@
+"""Host side of `vox_hybrid_*`: the engine for decoders that mix tokens with linear recurrences (HGRN2, mLSTM) and with
+sliding-window attention over a paged cache with pooled history, optionally looping a range of layers over shared weights.
+
+It reuses the plan / stream / hipGraph machinery of the other LM engines (`Qwen3Engine`): one pinned int32 plan block per
+step, decode steps captured per batch size.  Beyond the K / V pages that the worker hands out, every request holds one
+recurrent-state slot (`state` in the plan); the engine owns the slot arrays, the worker owns the free list.
+
+A step is ragged: `prefill(n_rows, n_req, ...)` takes prompt portions of any length next to single decoded tokens, `frame(batch,
+...)` is the one-row-per-request special case whose inputs feed back on the device.
+"""
+import ctypes
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional
+
+import torch
+
+from . import _native as N
+from .engine import Qwen3Engine
+
+MIXER_HGRN2, MIXER_POOLED_WINDOW_ATTN, MIXER_MLSTM = 0, 1, 2
+MIXER_KINDS = {"hgrn2": MIXER_HGRN2, "attention": MIXER_POOLED_WINDOW_ATTN, "mlstm": MIXER_MLSTM}
+
+
+@dataclass
+class MixerCfg:
+    kind: str                       # "hgrn2" | "attention" | "mlstm"
+    heads: int
+    dim: int
+    vdim: int
+    kv_heads: int = 0               # attention
+    window: int = 0                 # attention: tokens a position sees, itself included
+    pool: int = 0                   # attention: tokens per pooled block
+    rot_dims: int = 0
+    rot_base: float = 10000.0
+    rot_factor: float = 1.0         # linear position scaling: every rotary frequency is divided by it
+    scale: float = 1.0              # attention score scale
+    gate_cap: float = 0.0           # mLSTM: soft cap of the gate pre-activations
+    ff: int = 0                     # feed-forward width (0: none)
+
+    @property
+    def n_in(self) -> int:
+        """Rows of the fused input projection."""
+        h, d, v = self.heads, self.dim, self.vdim
+        if self.kind == "hgrn2":
+            return 2 * h * d + h * v
+        if self.kind == "attention":
+            return h * d + self.kv_heads * (d + v) + h
+        return 2 * h * d + 2 * h * v + 2 * h
+
+
+@dataclass
+class HybridCfg:
+    width: int
+    vocab: int
+    eps: float
+    layers: List[MixerCfg] = field(default_factory=list)
+    loop: Optional[tuple] = None    # (start, stop, times): layers start..stop-1 run `times` times in a row
+
+    def runs(self):
+        """[(layer index, loop_in)] in execution order; loop_in marks the first layer of every pass of the looped range."""
+        n = len(self.layers)
+        if not self.loop:
+            return [(i, False) for i in range(n)]
+        a, b, t = self.loop
+        out = [(i, False) for i in range(a)]
+        for _ in range(t):
+            out += [(i, i == a) for i in range(a, b)]
+        return out + [(i, False) for i in range(b, n)]
+
+
+class HybridLayerC(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("kind", "heads", "kv_heads", "dim", "vdim", "window", "pool", "rot_dims")] + \
+               [("scale", ctypes.c_float), ("gate_cap", ctypes.c_float), ("ff", ctypes.c_int32)] + \
+               [(n, ctypes.c_void_p) for n in ("norm1", "norm2", "w_in", "b_in", "w_out", "lower", "head_norm", "inv_freq",
+                                               "w_up", "w_down")]
+
+
+class HybridRunC(ctypes.Structure):
+    _fields_ = [("layer", ctypes.c_int32), ("loop_in", ctypes.c_int32), ("cache", ctypes.c_void_p), ("pool", ctypes.c_void_p),
+                ("state", ctypes.c_void_p)]
+
+
+class HybridConfigC(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("width", "vocab", "n_layers", "n_runs", "dtype", "page_size", "max_rows",
+                                              "max_batch", "max_out", "max_pages")] + [("eps", ctypes.c_float)]
+
+
+class HybridWeightsC(ctypes.Structure):
+    _fields_ = [("layers", ctypes.POINTER(HybridLayerC)), ("runs", ctypes.POINTER(HybridRunC))] + \
+               [(n, ctypes.c_void_p) for n in ("embedding", "loop_in", "head", "final_norm")]
+
+
+class HybridIO(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_void_p) for n in ("pos", "row_req", "page", "slot", "req_rows", "req_state", "page_table")] + \
+               [("pt_stride", ctypes.c_int32)] + \
+               [(n, ctypes.c_void_p) for n in ("out_rows", "logits", "trace", "input_ids", "out_ids", "rng_offset")]
+
+
+def rotary_frequencies(rot_dims: int, base: float, factor: float) -> torch.Tensor:
+    """f_i = base^(-2i/rot_dims) / factor, i < rot_dims/2, in fp32 arithmetic."""
+    i = torch.arange(rot_dims // 2, dtype=torch.float32)
+    return torch.pow(torch.tensor(base, dtype=torch.float32), -(2.0 * i) / rot_dims) / factor
+
+
+class HybridEngine(Qwen3Engine):
+    """`weights`: {"embedding", "head", "final_norm", "loop_in" (or None), "layers": [per layer dict with norm1, norm2, w_in,
+    b_in, w_out, lower, head_norm, w_up, w_down]} — matrices in any float dtype (stored as the engine's dtype), vectors
+    stored as fp32.  dtype: torch.bfloat16 or torch.float32."""
+
+    needs_state_slots = True
+
+    def __init__(self, cfg: HybridCfg, weights: Dict, dtype=torch.bfloat16, max_batch=8, page_size=128, max_pages=256,
+                 max_seq_len=4096, max_prefill_rows=1024, max_out=None, state_slots=None, device="cuda"):
+        if dtype not in (torch.bfloat16, torch.float32):
+            raise ValueError(f"HybridEngine: dtype {dtype} (bfloat16 or float32)")
+        self.cfg, self.device, self.dtype = cfg, torch.device(device), dtype
+        self.max_batch, self.page_size, self.max_pages, self.max_seq_len = max_batch, page_size, max_pages, max_seq_len
+        self.max_rows = max(max_prefill_rows, max_batch)
+        self.max_out = max(max_out or max_batch, max_batch)
+        self.state_slots = state_slots or max_batch
+        self.L, self.ctx = N.lib(), N.ctx()
+        L, vp, ci = self.L, ctypes.c_void_p, ctypes.c_int
+        L.vox_hybrid_create.restype, L.vox_hybrid_create.argtypes = ci, [vp, ctypes.POINTER(HybridConfigC), ctypes.POINTER(HybridWeightsC), ctypes.POINTER(vp)]
+        L.vox_hybrid_destroy.restype, L.vox_hybrid_destroy.argtypes = None, [vp]
+        L.vox_hybrid_step.restype, L.vox_hybrid_step.argtypes = ci, [vp, vp, ctypes.POINTER(HybridIO), vp, ci, ci, ci, ctypes.POINTER(N.SamplingCfg), ctypes.c_uint64, ci]
+        dev = self.device
+        self._keep = []
+
+        def mat(t):
+            if t is None:
+                return None
+            self._keep.append(t.to(dev, dtype).contiguous())
+            return self._keep[-1].data_ptr()
+
+        def vec(t):
+            if t is None:
+                return None
+            self._keep.append(t.to(dev, torch.float32).contiguous())
+            return self._keep[-1].data_ptr()
+
+        W = cfg.width
+        larr = (HybridLayerC * len(cfg.layers))()
+        for i, (m, lw) in enumerate(zip(cfg.layers, weights["layers"])):
+            assert tuple(lw["w_in"].shape) == (m.n_in, W), (i, tuple(lw["w_in"].shape), m.n_in)
+            assert tuple(lw["w_out"].shape) == (W, m.heads * m.vdim), (i, tuple(lw["w_out"].shape))
+            c = larr[i]
+            c.kind, c.heads, c.kv_heads, c.dim, c.vdim = MIXER_KINDS[m.kind], m.heads, m.kv_heads, m.dim, m.vdim
+            c.window, c.pool, c.rot_dims, c.scale, c.gate_cap, c.ff = m.window, m.pool, m.rot_dims, m.scale, m.gate_cap, m.ff
+            c.norm1, c.norm2 = vec(lw["norm1"]), vec(lw.get("norm2"))
+            c.w_in, c.b_in, c.w_out = mat(lw["w_in"]), vec(lw.get("b_in")), mat(lw["w_out"])
+            c.lower, c.head_norm = vec(lw.get("lower")), vec(lw.get("head_norm"))
+            c.inv_freq = vec(rotary_frequencies(m.rot_dims, m.rot_base, m.rot_factor)) if m.kind == "attention" and m.rot_dims else None
+            c.w_up, c.w_down = mat(lw.get("w_up")), mat(lw.get("w_down"))
+        runs = cfg.runs()
+        rarr = (HybridRunC * len(runs))()
+        self.caches, self.pools, self.states = [], [], []
+        for j, (li, loop_in) in enumerate(runs):
+            m = cfg.layers[li]
+            rarr[j].layer, rarr[j].loop_in = li, int(loop_in)
+            if m.kind == "attention":
+                kv = torch.zeros(max_pages * page_size * m.kv_heads * (m.dim + m.vdim), dtype=dtype, device=dev)
+                pool = torch.zeros(max_pages, (page_size - 1) // m.pool + 1, m.kv_heads, m.dim + m.vdim, dtype=torch.float32, device=dev)
+                self.caches.append(kv); self.pools.append(pool)
+                rarr[j].cache, rarr[j].pool = kv.data_ptr(), pool.data_ptr()
+            else:
+                per = m.dim * m.vdim + (m.dim + 1 if m.kind == "mlstm" else 0)
+                st = torch.zeros(self.state_slots, m.heads, per, dtype=torch.float32, device=dev)
+                self.states.append(st)
+                rarr[j].state = st.data_ptr()
+        self.n_runs = len(runs)
+        cc = HybridConfigC(W, cfg.vocab, len(cfg.layers), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
+                           max_batch, self.max_out, max_pages, cfg.eps)
+        cw = HybridWeightsC(ctypes.cast(larr, ctypes.POINTER(HybridLayerC)), ctypes.cast(rarr, ctypes.POINTER(HybridRunC)),
+                            mat(weights["embedding"]), mat(weights.get("loop_in")), mat(weights["head"]), vec(weights["final_norm"]))
+        self._larr, self._rarr = larr, rarr
+        h = ctypes.c_void_p()
+        N.check(L.vox_hybrid_create(self.ctx, ctypes.byref(cc), ctypes.byref(cw), ctypes.byref(h)))
+        self.h = h
+        i32 = dict(dtype=torch.int32, device=dev)
+        R = self.max_rows
+        self.input_ids = torch.zeros(max_batch, 1, **i32)
+        self.row_ids = torch.zeros(R, 1, **i32)
+        self.row_masks = torch.zeros(R, dtype=torch.uint8, device=dev)           # (unused: kept for the worker's staging code)
+        self.pt_stride = (max_seq_len + page_size - 1) // page_size + 1
+        self._plan_layout, off = {}, 0
+        for name, n in (("pos", R), ("kvlen", R), ("page", R), ("slot", R), ("q_req", R), ("last_rows", self.max_out),
+                        ("indptr", max_batch + 1), ("indices", max_pages), ("ptab", max_batch * self.pt_stride),
+                        ("req_rows", max_batch + 1), ("state", max_batch)):
+            self._plan_layout[name] = (off, n)
+            off += n
+        self.plan_dev = torch.zeros(off, **i32)
+        self._init_plan_host(off)
+        self.out_ids = torch.zeros(max_batch, **i32)
+        self.out_logits = torch.zeros(self.max_out, cfg.vocab, dtype=torch.float32, device=dev)
+        self.rng_offset = torch.zeros(1, dtype=torch.int64, device=dev)
+        self.trace = None
+        self.rep_cache = None
+        self._graphs, self.keep_hidden = {}, False
+
+    def enable_trace(self):
+        """Keep the residual stream after every layer run of the next steps: trace[run, row, :]."""
+        if self.trace is None:
+            self.trace = torch.zeros(self.n_runs, self.max_rows, self.cfg.width, dtype=torch.float32, device=self.device)
+            self._drop_graphs()
+        return self.trace
+
+    def _io(self):
+        return HybridIO(self._pd("pos").data_ptr(), self._pd("q_req").data_ptr(), self._pd("page").data_ptr(),
+                        self._pd("slot").data_ptr(), self._pd("req_rows").data_ptr(), self._pd("state").data_ptr(),
+                        self._pd("ptab").data_ptr(), self.pt_stride, self._pd("last_rows").data_ptr(), self.out_logits.data_ptr(),
+                        self.trace.data_ptr() if self.trace is not None else None, self.input_ids.data_ptr(),
+                        self.out_ids.data_ptr(), self.rng_offset.data_ptr())
+
+    def _mutable_state(self):
+        # a decode step advances the recurrent states and appends K / V: the warm-up run before a capture must leave no trace
+        return [self.input_ids, self.rng_offset] + self.states
+
+    def _native_frame(self, io, st, batch, bucket, sampling, seed, feedback):
+        N.check(self.L.vox_hybrid_step(self.h, st, ctypes.byref(io), self.input_ids.data_ptr(), batch, batch, batch,
+                                       ctypes.byref(sampling), seed, int(feedback)))
+
+    def _native_destroy(self):
+        self.L.vox_hybrid_destroy(self.h)
+
+    def step(self, n_rows, n_req, n_out=None, sampling=None, seed=0, feedback=True, sample=True):
+        """One ragged step, eagerly: rows staged in row_ids + plan arrays.  n_out rows (plan `last_rows`) get logits in
+        out_logits[:n_out]; with `sample`, requests 0..n_req-1 are sampled from output rows 0..n_req-1."""
+        n_out = n_req if n_out is None else n_out
+        io = self._io()
+        sc = ctypes.byref(sampling or self.sampling_cfg()) if sample else None
+        self._log_launch("prefill", (n_rows, n_req, n_out), n_req)
+        N.check(self.L.vox_hybrid_step(self.h, N.stream(), ctypes.byref(io), self.row_ids.data_ptr(), n_rows, n_req, n_out, sc, seed,
+                                       int(feedback and sample)))
+
+    def _prefill_on_stream(self, n_rows, n_req, max_kvlen, sampling, seed, feedback):
+        if n_req == 0:
+            raise N.VoxError("HybridEngine: a step without requests")
+        io = self._io()
+        N.check(self.L.vox_hybrid_step(self.h, N.stream(), ctypes.byref(io), self.row_ids.data_ptr(), n_rows, n_req, n_req,
+                                       ctypes.byref(sampling), seed, int(feedback)))
+
+    @staticmethod
+    def sampling_cfg(greedy=True, top_k=0, top_p=1.0, min_p=0.0, temperature=1.0, repetition_penalty=1.0):
+        return N.SamplingCfg(int(greedy), int(top_k or 0), float(1.0 if top_p is None else top_p), float(min_p or 0.0),
+                             float(temperature), 1.0)

@@ -159,6 +159,35 @@ def _orpheus(model_name, device="cuda:0", weights=None, codec_weights=None, chec
     return OrpheusModel(model_name, weights, codec_weights, config=config, device=device, **kw)
 
 
+@register_model("sirodra")
+def _sirodra(model_name, device="cuda:0", weights=None, checkpoint_dir=None, synthetic=False, config=None, **kw):
+    """Text-only hybrid-mixer LM.  checkpoint_dir: a folder with config.json + model.safetensors; synthetic: random weights for
+    `config` (a HybridCfg)."""
+    from .sirodra import SirodraModel, synth_weights
+    kw.pop("detokenize_interval", None)
+    if "max_num_pages" in kw and "max_seq_len" not in kw:
+        kw["max_seq_len"] = min(kw["max_num_pages"] * kw.get("page_size", 128), 1 << 16)
+    if weights is None and checkpoint_dir is not None:
+        return SirodraModel.from_checkpoint(checkpoint_dir, model_name=model_name, device=device, **kw)
+    if config is None:
+        raise FileNotFoundError("no checkpoint_dir given: pass checkpoint_dir=... or config=... with weights / synthetic=True")
+    if weights is None:
+        if not synthetic:
+            raise FileNotFoundError("no checkpoint_dir given (offline box): pass checkpoint_dir=... or synthetic=True")
+        weights = synth_weights(config)
+    return SirodraModel(model_name, weights, config, device=device, **kw)
+
+
+def load_checkpoint_dir(path: str, device: str = "cuda:0", **kw):
+    """A local checkpoint folder whose config.json names its architecture: the registry entry of that name loads it."""
+    import json
+    with open(os.path.join(path, "config.json")) as f:
+        arch = json.load(f).get("architecture")
+    if not arch:
+        raise ValueError(f"{path}/config.json names no architecture")
+    return get_model_class(arch)(arch, device=device, checkpoint_dir=path, **kw)
+
+
 def load_model(model_name: str, device: str = "cuda", top_p=None, top_k=None, min_p=None, temperature=None,
                max_tokens=None, repetition_penalty=None, repetition_window=None, cfg_scale=None, greedy=False,
                enable_torch_compile=False, audio_decoder_device=None, detokenize_interval=None, **kw):

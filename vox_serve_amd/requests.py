@@ -56,6 +56,13 @@ class Request:
     prefill_ready: bool = False
     eos_injected: bool = False
 
+    # ragged engines (recurrent-state models): the state slot the request holds, how much of its prompt has run, how many prompt
+    # tokens the next step may take (None: all that is left), and whether more prompt tokens will still be appended
+    state_slot: int = None
+    prefill_cursor: int = 0
+    step_budget: int = None
+    prompt_open: bool = False
+
     chunk_send_timestamps: List[float] = field(default_factory=list)
     chunk_durations: List[float] = field(default_factory=list)
 

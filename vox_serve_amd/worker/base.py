@@ -46,7 +46,7 @@ class ModelWorker:
                  cfg_scale: float = None, greedy: bool = False, enable_nvtx: bool = False,
                  enable_torch_compile: bool = False, detokenizer_device: Optional[str] = None, dp_rank: int = 0,
                  dp_size: int = 1, detokenize_interval: int = None, model=None, device: str = "cuda:0", seed: int = 0,
-                 exact_rows: Optional[int] = None):
+                 exact_rows: Optional[int] = None, prefill_chunk_tokens: Optional[int] = None):
         if exact_rows is not None:
             # rows up to which the wave64 VALU kernels are used (include/voxhip.h: vox_ctx_set_exact_rows): must precede the engines' creation
             from .. import _native as _N
@@ -77,6 +77,13 @@ class ModelWorker:
         self.empty_pages = queue.Queue()
         for i in range(max_num_pages):
             self.empty_pages.put(i)
+        # models with recurrent layers hold one state slot per live request next to their K / V pages: the engine owns the slot
+        # arrays, this free list hands them out at admission and takes them back in free_kv_cache
+        self.empty_state_slots = queue.Queue()
+        for i in range(int(getattr(getattr(model, "engine", None), "state_slots", 0) or 0)):
+            self.empty_state_slots.put(i)
+        # prompts may be prefilled in portions (ragged engines only): at most this many prompt tokens of a request per step
+        self.prefill_chunk_tokens = prefill_chunk_tokens
         self.needs_watermarking = getattr(model, "needs_watermarking", False)
         self.has_depth_transformer = getattr(model, "has_depth_transformer", False)
         self.async_scheduling = False   # set by a scheduler running the reference's async loop (scheduler/base.py:166-221)
@@ -140,30 +147,57 @@ class ModelWorker:
                                           or any(getattr(r, "is_input_streaming", False) for r in lm_requests)):
             self.drain()             # this step reads per-request host state (restaging): finish the deferred update first
         ps = self.page_size
-        # admission: preprocess the new prompts (once) and count the pages this step takes before touching any KV state
-        need = 0
+        ragged = self._ragged()
+        # admission: preprocess the new prompts (once) and count the pages / state slots this step takes before touching any state
+        need, need_slots, take = 0, 0, {}
         for req in lm_requests:
             if not req.done_lm_prefill:
                 self._preprocess_request(req)
-                need += (len(req.input_tokens) + ps - 1) // ps
+                cur = int(getattr(req, "prefill_cursor", 0) or 0) if ragged else 0
+                n = len(req.input_tokens) - cur
+                if ragged:
+                    # a portion: the request's own budget for this step, the worker's chunk size, the engine's row capacity
+                    for cap in (getattr(req, "step_budget", None), self.prefill_chunk_tokens,
+                                self.model.engine.max_rows - (len(lm_requests) - 1)):
+                        if cap:
+                            n = min(n, int(cap))
+                    if n < 1:
+                        raise ValueError(f"request {req.request_id}: no prompt tokens to run")
+                    if getattr(req, "state_slot", None) is None and getattr(self.model.engine, "state_slots", 0):
+                        need_slots += 1
+                take[req.request_id] = (cur, n)
+                need += (cur + n + ps - 1) // ps - (len(req.kv_pages or []) if cur else 0)
             elif req.kv_last_page_len + 1 > ps:
                 need += 1
         if need > self.empty_pages.qsize():
             raise OutOfPages(f"step needs {need} KV pages, {self.empty_pages.qsize()} free")
+        if need_slots > self.empty_state_slots.qsize():
+            raise OutOfPages(f"step needs {need_slots} state slots, {self.empty_state_slots.qsize()} free")
         for req in lm_requests:
             if not req.done_lm_prefill:
-                n = len(req.input_tokens)
-                input_ids_list.append(req.input_tokens)
-                position_ids_list.extend(range(n))
+                cur, n = take[req.request_id]
+                input_ids_list.append(req.input_tokens[cur:cur + n] if ragged else req.input_tokens)
+                position_ids_list.extend(range(cur, cur + n))
                 feats.append(req.input_features)
                 masks.append(req.input_masks)
                 reps.append(req.repetition_cache)
-                req.kv_token_len = n
-                req.kv_pages = [self.empty_pages.get_nowait() for _ in range((n + ps - 1) // ps)]
-                req.kv_last_page_len = n % ps or ps
+                req.kv_token_len = cur + n
+                if not cur:
+                    req.kv_pages = []
+                req.kv_pages.extend(self.empty_pages.get_nowait() for _ in range((cur + n + ps - 1) // ps - len(req.kv_pages)))
+                req.kv_last_page_len = (cur + n) % ps or ps
                 qo_indptr.append(qo_indptr[-1] + n)
-                req.next_position_id = n + 1          # quirk Q1 (worker/base.py:299)
-                req.done_lm_prefill = True
+                if ragged:
+                    if getattr(req, "state_slot", None) is None and getattr(self.model.engine, "state_slots", 0):
+                        req.state_slot = self.empty_state_slots.get_nowait()
+                    req.prefill_cursor = cur + n
+                    # the prompt is done when its last token has run, unless more of it is still to come (prompt_open)
+                    if cur + n == len(req.input_tokens) and not getattr(req, "prompt_open", False):
+                        req.done_lm_prefill = True
+                    req.next_position_id = cur + n      # positions are the tokens' indices in the sequence
+                else:
+                    req.next_position_id = n + 1          # quirk Q1 (worker/base.py:299)
+                    req.done_lm_prefill = True
             else:
                 if req.is_input_streaming:
                     self._inject_streaming_text_token(req)
@@ -205,6 +239,10 @@ class ModelWorker:
                 "paged_kv_last_page_len": paged_kv_last_page_len, "input_ids": input_ids, "position_ids": position_ids,
                 "input_features": input_features, "input_masks": input_masks, "repetition_cache": repetition_cache,
                 "is_prefill": is_prefill, "prefill_flags": prefill_flags}
+
+    def _ragged(self) -> bool:
+        """The engine takes ragged steps (prompt portions of any length next to decode rows) and keeps per-request state slots."""
+        return bool(getattr(getattr(self.model, "engine", None), "needs_state_slots", False))
 
     def _preprocess_request(self, req: Request) -> None:
         """model.preprocess -> request fields (worker/base.py:246-270), once per request."""
@@ -278,6 +316,8 @@ class ModelWorker:
             return None
         e = self.model.engine
         n_rows, n_req = int(lm_inputs["input_ids"].shape[0]), len(requests)
+        if self._ragged():
+            return self._run_ragged_step(requests, lm_inputs)
         if n_rows > e.max_rows or n_req > e.max_batch:
             if n_req != 1:
                 # a prompt (plus the decode rows piggy-backed onto its step) that does not fit the engine's row capacity:
@@ -307,6 +347,46 @@ class ModelWorker:
         self.nvtx_range_pop()
         self.nvtx_range_pop()
         return task
+
+    def _run_ragged_step(self, requests: List[Request], lm_inputs: LMInputs):
+        """One step of a ragged engine: every request's rows (a prompt portion or one decoded token) in one launch.  Requests whose
+        prompt ended in this step are sampled and updated; a portion in the middle of a prompt only leaves its K / V and state.
+        `lm_inputs["logit_rows"]` (optional): rows of the step whose logits are kept in engine.out_logits behind the requests'
+        last rows (teacher-forced scoring)."""
+        e = self.model.engine
+        self.drain()
+        n_rows, n_req = int(lm_inputs["input_ids"].shape[0]), len(requests)
+        if n_rows > e.max_rows or n_req > e.max_batch:
+            raise ValueError(f"step of {n_rows} rows / {n_req} requests exceeds the engine ({e.max_rows} / {e.max_batch})")
+        self.nvtx_range_push(f"lm_prefill_bs{n_req}")
+        q_req, kvlen, page, slot = self._token_plan(lm_inputs)
+        e.row_ids[:n_rows].copy_(lm_inputs["input_ids"].to(torch.int32).view(n_rows, -1)[:, :1])
+        qo = lm_inputs["qo_indptr"]
+        out_rows = [q - 1 for q in qo[1:]] + [int(r) for r in (lm_inputs.get("logit_rows") or [])]
+        if len(out_rows) > e.max_out:
+            raise ValueError(f"{len(out_rows)} logit rows exceed the engine's {e.max_out}")
+        e.upload_plan(pos=lm_inputs["position_ids"].numpy(), kvlen=kvlen, page=page, slot=slot, q_req=q_req, last_rows=out_rows,
+                      indptr=lm_inputs["paged_kv_indptr"], indices=lm_inputs["paged_kv_indices"], req_rows=qo,
+                      state=[int(getattr(r, "state_slot", 0) or 0) for r in requests])
+        ended = [i for i, r in enumerate(requests) if r.done_lm_prefill]
+        e.step(n_rows, n_req, n_out=len(out_rows), sampling=self._sampling(), seed=self.seed, feedback=True, sample=bool(ended))
+        self.nvtx_range_pop()
+        if ended:
+            out = e.out_ids[:n_req].cpu().to(torch.long)
+            self._update_requests([requests[i] for i in ended], out[ended].view(len(ended), -1), None, None)
+        # the engine's decode inputs hold this step's picks in ITS request order: valid for the next decode step only if that step
+        # has exactly these requests (all of them sampled)
+        self._resident = [r.request_id for r in requests] if len(ended) == n_req else None
+        self._resident_reqs = []
+        return None
+
+    def _state_plan(self, requests: List[Request]) -> dict:
+        """Plan arrays of a decode step that only ragged engines read: one row per request, its state slot."""
+        if not self._ragged():
+            return {}
+        B = len(requests)
+        return {"q_req": list(range(B)), "req_rows": list(range(B + 1)), "last_rows": list(range(B)),
+                "state": [int(getattr(r, "state_slot", 0) or 0) for r in requests]}
 
     @staticmethod
     def _slice_inputs(lm_inputs: LMInputs, lo: int, hi: int) -> LMInputs:
@@ -390,7 +470,7 @@ class ModelWorker:
             self._stage_repetition(requests, e)
         e.upload_plan(pos=lm_inputs["position_ids"].numpy(), kvlen=[r.kv_token_len for r in requests],
                       page=[r.kv_pages[-1] for r in requests], slot=[r.kv_last_page_len - 1 for r in requests],
-                      indptr=lm_inputs["paged_kv_indptr"], indices=lm_inputs["paged_kv_indices"])
+                      indptr=lm_inputs["paged_kv_indptr"], indices=lm_inputs["paged_kv_indices"], **self._state_plan(requests))
         self.nvtx_range_push("cuda_graph_replay")                # one hipGraph: talker + sampling + the whole depth loop
         e.frame(B, max(r.kv_token_len for r in requests), self._sampling(), seed=self.seed, feedback=True)
         self.nvtx_range_pop()
@@ -741,6 +821,9 @@ class ModelWorker:
             request.kv_pages = []
             request.kv_token_len = 0
             request.kv_last_page_len = 0
+        if getattr(request, "state_slot", None) is not None:
+            self.empty_state_slots.put(request.state_slot)      # the next owner starts from zero: its first row is at position 0
+            request.state_slot = None
         dc = getattr(request, "decoder_cache", None)
         if dc is not None and hasattr(self.model, "audio_decoder") and hasattr(self.model.audio_decoder, "release_cache"):
             self.model.audio_decoder.release_cache(dc)

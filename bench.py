@@ -740,8 +740,15 @@ def main():
     ap.add_argument("--serving-frames", type=int, default=250, help="frames per request of the serving-path jobs (SURVEY 8d: 250)")
     ap.add_argument("--exact-rows", type=int, default=None, help="rows up to which linears use the wave64 VALU kernels instead of the "
                     "matrix cores (library default 2; 1..8).  Every setting is bit-exact against the oracle under the same policy")
+    ap.add_argument("--sirodra", action="store_true", help="instead of the default workload: prefill / decode throughput of the hybrid-mixer "
+                    "engine (Sirodra layer pattern, random weights) beside the single-stack LM engine at equal width and depth "
+                    "(tools/bench_sirodra.py); prints that comparison as one JSON line")
     args = ap.parse_args()
 
+    if args.sirodra:
+        from tools.bench_sirodra import run as run_sirodra
+        print(json.dumps(run_sirodra(steps=min(args.steps, 50), warmup=min(args.warmup, 10))))
+        return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(spawn_ranks(args))
     rank = int(os.environ.get("RANK", "0"))

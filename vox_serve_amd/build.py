@@ -36,9 +36,13 @@ def build(force: bool = False, verbose: bool = False) -> str:
     objs = []
     procs = []
     os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
+    hdrs = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")] + [os.path.join(HERE, "..", "include", "voxhip.h"), __file__]
+    newest_hdr = max(os.path.getmtime(h) for h in hdrs)
     for s in srcs:
         o = os.path.join(HERE, "build", os.path.basename(s) + ".o")
         objs.append(o)
+        if not force and os.path.exists(o) and os.path.getmtime(o) > max(os.path.getmtime(s), newest_hdr):
+            continue                    # this object is newer than its source and every header: keep it
         procs.append((s, subprocess.Popen([_hipcc(), *FLAGS, "-c", s, "-o", o], stdout=subprocess.PIPE,
                                           stderr=subprocess.STDOUT)))
     for s, p in procs:

@@ -239,29 +239,37 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
     }
 }
 
-// 1..8 rows (decode): one wave per output column streams its weight row once, 16 bytes per lane and request; lanes own
-// k-chunks c, c + 64, ...; butterfly at the end.
+// 1..8 rows (decode): a wave streams CPW weight rows (output columns) at once, 16 bytes per lane and request, against one read of
+// the activations; lanes own k-chunks c, c + 64, ...; butterfly at the end.  The order of each output's sum depends on K only.
+#define HB_GEMV_CPW 4
 template <typename T, int MR, int EPI>
 __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const T* Wt, const float* bias, float* C, long ldc, int M, int N,
                                                  int K) {
-    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (n >= N) return;
+    const int lane = threadIdx.x & 63, n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * HB_GEMV_CPW;
+    if (n0 >= N) return;
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
-    float acc[MR];
+    float acc[MR][HB_GEMV_CPW];
 #pragma unroll
-    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
-    const T* wr = Wt + (size_t)n * K;
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int j = 0; j < HB_GEMV_CPW; ++j) acc[m][j] = 0.f;
+    const T* wr[HB_GEMV_CPW];
+#pragma unroll
+    for (int j = 0; j < HB_GEMV_CPW; ++j) wr[j] = Wt + (size_t)(n0 + j < N ? n0 + j : N - 1) * K;
     const bool vec = (K % CH == 0) && ((((size_t)Wt) & 15) == 0) && (lda % 4 == 0) && ((((size_t)A) & 15) == 0);
     if (vec) {
         for (int k = lane * CH; k < K; k += 64 * CH) {
-            float w[CH];
-            if (sizeof(T) == 2) {
-                const uint4 u = *(const uint4*)(wr + k);
-                w[0] = bflo(u.x); w[1] = bfhi(u.x); w[2] = bflo(u.y); w[3] = bfhi(u.y);
-                if (CH == 8) { w[4] = bflo(u.z); w[5] = bfhi(u.z); w[6] = bflo(u.w); w[7] = bfhi(u.w); }
-            } else {
-                const float4 u = *(const float4*)(wr + k);
-                w[0] = u.x; w[1] = u.y; w[2] = u.z; w[3] = u.w;
+            float w[HB_GEMV_CPW][CH];
+#pragma unroll
+            for (int j = 0; j < HB_GEMV_CPW; ++j) {
+                if (sizeof(T) == 2) {
+                    const uint4 u = *(const uint4*)(wr[j] + k);
+                    w[j][0] = bflo(u.x); w[j][1] = bfhi(u.x); w[j][2] = bflo(u.y); w[j][3] = bfhi(u.y);
+                    if (CH == 8) { w[j][4] = bflo(u.z); w[j][5] = bfhi(u.z); w[j][6] = bflo(u.w); w[j][7] = bfhi(u.w); }
+                } else {
+                    const float4 u = *(const float4*)(wr[j] + k);
+                    w[j][0] = u.x; w[j][1] = u.y; w[j][2] = u.z; w[j][3] = u.w;
+                }
             }
 #pragma unroll
             for (int m = 0; m < MR; ++m) {
@@ -269,28 +277,36 @@ __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const
                 const float* xr = A + (size_t)m * lda + k;
 #pragma unroll
                 for (int e = 0; e < CH; e += 4) {
-                    const float4 x = *(const float4*)(xr + e);
-                    acc[m] = fmaf(w[e], hb_operand<T>(x.x), acc[m]);
-                    acc[m] = fmaf(w[e + 1], hb_operand<T>(x.y), acc[m]);
-                    acc[m] = fmaf(w[e + 2], hb_operand<T>(x.z), acc[m]);
-                    acc[m] = fmaf(w[e + 3], hb_operand<T>(x.w), acc[m]);
+                    const float4 x4 = *(const float4*)(xr + e);
+                    const float x[4] = {hb_operand<T>(x4.x), hb_operand<T>(x4.y), hb_operand<T>(x4.z), hb_operand<T>(x4.w)};
+#pragma unroll
+                    for (int j = 0; j < HB_GEMV_CPW; ++j) {
+                        acc[m][j] = fmaf(w[j][e], x[0], acc[m][j]);
+                        acc[m][j] = fmaf(w[j][e + 1], x[1], acc[m][j]);
+                        acc[m][j] = fmaf(w[j][e + 2], x[2], acc[m][j]);
+                        acc[m][j] = fmaf(w[j][e + 3], x[3], acc[m][j]);
+                    }
                 }
             }
         }
     } else {
         for (int k = lane; k < K; k += 64) {
-            const float w = hb_ld(wr + k);
 #pragma unroll
-            for (int m = 0; m < MR; ++m)
-                if (m < M) acc[m] = fmaf(w, hb_operand<T>(A[(size_t)m * lda + k]), acc[m]);
+            for (int j = 0; j < HB_GEMV_CPW; ++j) {
+                const float w = hb_ld(wr[j] + k);
+#pragma unroll
+                for (int m = 0; m < MR; ++m)
+                    if (m < M) acc[m][j] = fmaf(w, hb_operand<T>(A[(size_t)m * lda + k]), acc[m][j]);
+            }
         }
     }
-    const float b = bias ? bias[n] : 0.f;
 #pragma unroll
-    for (int m = 0; m < MR; ++m) {
-        const float s = hb_wave_sum(acc[m]);
-        if (m < M && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n, s, b);
-    }
+    for (int m = 0; m < MR; ++m)
+#pragma unroll
+        for (int j = 0; j < HB_GEMV_CPW; ++j) {
+            const float sum = hb_wave_sum(acc[m][j]);
+            if (m < M && n0 + j < N && lane == 0) hb_epilogue<EPI>(C + (size_t)m * ldc + n0 + j, sum, bias ? bias[n0 + j] : 0.f);
+        }
 }
 
 template <typename T, int EPI>
@@ -311,7 +327,7 @@ int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const float* W, cons
 template <typename T, int EPI>
 int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
     if (M <= 0 || N <= 0) return VOX_OK;
-    const dim3 g((N + 3) / 4), b(256);
+    const dim3 g((N + 4 * HB_GEMV_CPW - 1) / (4 * HB_GEMV_CPW)), b(256);
     if (M == 1) hipLaunchKernelGGL((k_hb_gemv<T, 1, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
     else if (M == 2) hipLaunchKernelGGL((k_hb_gemv<T, 2, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
     else if (M <= 4) hipLaunchKernelGGL((k_hb_gemv<T, 4, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
@@ -326,104 +342,131 @@ int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const
     return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K);
 }
 
-// ---- HGRN2: S_t = diag(f_t) S_{t-1} + (1 - f_t) v_t^T,  o_t = S_t^T q_t ---------------------------------------------------
-// proj row = [q (H*dim) | f (H*dim) | v (H*vdim)] pre-activation (bias already added).  One wave per (request, head, 64 value
-// columns): the state tile lives in LDS for the whole portion and goes back to its slot at the end.
-__global__ __launch_bounds__(64) void k_hb_hgrn2_scan(const float* proj, long ldp, float* out, long ldo, const float* lower, float* state,
-                                                      const int* req_rows, const int* req_state, const int* pos, int H, int dim, int vdim) {
-    extern __shared__ float sm[];
-    float* S = sm;                 // [dim][64]
-    float* fs = sm + dim * 64;     // [dim]
-    float* qs = fs + dim;          // [dim]
-    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, c = blockIdx.z * 64 + lane;
+// ---- linear recurrences ------------------------------------------------------------------------------------------------------
+// One block per (request, head, 64 value columns); wave w owns DPW consecutive key dims of those columns and keeps its part of
+// the state in registers for the whole portion (loaded from the request's slot unless the portion starts the sequence, written
+// back at the end).  Per token: the block stages the token's per-dim factors in LDS, every thread updates its DPW state values
+// and accumulates its partial output, the partials of the waves are added in wave order.  The order of every sum depends on
+// (dim, DPW) only, never on how the tokens are cut into steps.
+#define HB_SCAN_MAX_WAVES 16
+
+// HGRN2: S_t = diag(f_t) S_{t-1} + (1 - f_t) v_t^T,  o_t = S_t^T q_t.
+// proj row = [q (H*dim) | f (H*dim) | v (H*vdim)] pre-activation (bias already added).
+template <int DPW>
+__global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_hgrn2_scan(const float* proj, long ldp, float* out, long ldo, const float* lower,
+                                                                          float* state, const int* req_rows, const int* req_state,
+                                                                          const int* pos, int H, int dim, int vdim) {
+    __shared__ float fs[HB_SCAN_MAX_WAVES * DPW], qs[HB_SCAN_MAX_WAVES * DPW], part[HB_SCAN_MAX_WAVES][64];
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.z * 64 + lane;
+    const int nw = blockDim.x >> 6, d0 = w * DPW;
     const int rs = req_rows[r], re = req_rows[r + 1];
     if (rs >= re) return;
     const bool ok = c < vdim, fresh = pos[rs] == 0;
     float* St = state + ((size_t)req_state[r] * H + h) * dim * vdim;
-    for (int d = 0; d < dim; ++d) S[d * 64 + lane] = (ok && !fresh) ? St[(size_t)d * vdim + c] : 0.f;
+    float S[DPW];
+#pragma unroll
+    for (int i = 0; i < DPW; ++i) S[i] = (ok && !fresh && d0 + i < dim) ? St[(size_t)(d0 + i) * vdim + c] : 0.f;
     for (int t = rs; t < re; ++t) {
         const float* p = proj + (size_t)t * ldp;
-        for (int d = lane; d < dim; d += 64) {
-            const float qv = p[h * dim + d];
-            qs[d] = qv * hb_sigmoid(qv);
-            const float lo = lower[h * dim + d];
-            fs[d] = lo + (1.0f - lo) * hb_sigmoid(p[H * dim + h * dim + d]);
+        for (int d = threadIdx.x; d < nw * DPW; d += blockDim.x) {
+            float q = 0.f, f = 0.f;
+            if (d < dim) {
+                const float qv = p[h * dim + d], lo = lower[h * dim + d];
+                q = qv * hb_sigmoid(qv);
+                f = lo + (1.0f - lo) * hb_sigmoid(p[H * dim + h * dim + d]);
+            }
+            qs[d] = q;
+            fs[d] = f;
         }
-        __syncthreads();
         const float v = ok ? p[2 * H * dim + h * vdim + c] : 0.f;
-        float o = 0.f;
-        for (int d = 0; d < dim; ++d) {
-            const float f = fs[d];
-            const float s = f * S[d * 64 + lane] + (1.0f - f) * v;
-            S[d * 64 + lane] = s;
-            o = fmaf(s, qs[d], o);
-        }
-        if (ok) out[(size_t)t * ldo + h * vdim + c] = o;
         __syncthreads();
+        float o = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPW; ++i) {
+            const float f = fs[d0 + i];
+            const float sv = f * S[i] + (1.0f - f) * v;
+            S[i] = sv;
+            o = fmaf(sv, qs[d0 + i], o);
+        }
+        part[w][lane] = o;
+        __syncthreads();
+        if (w == 0 && ok) {
+            float sum = part[0][lane];
+            for (int k = 1; k < nw; ++k) sum += part[k][lane];
+            out[(size_t)t * ldo + h * vdim + c] = sum;
+        }
     }
     if (ok)
-        for (int d = 0; d < dim; ++d) St[(size_t)d * vdim + c] = S[d * 64 + lane];
+#pragma unroll
+        for (int i = 0; i < DPW; ++i)
+            if (d0 + i < dim) St[(size_t)(d0 + i) * vdim + c] = S[i];
 }
 
-// ---- mLSTM with the running-maximum stabiliser -------------------------------------------------------------------------------
+// mLSTM with the running-maximum stabiliser.
 // proj row = [q (H*dim) | k (H*dim) | v (H*vdim) | g (H*vdim) | i (H) | f (H)].  State per (slot, head): S [dim][vdim], n [dim], m.
-// Every value tile keeps its own copy of n and m (same arithmetic, same order); tile 0 writes them back.
-__global__ __launch_bounds__(64) void k_hb_mlstm_scan(const float* proj, long ldp, float* out, long ldo, float* state, const int* req_rows,
-                                                      const int* req_state, const int* pos, int H, int dim, int vdim, float cap) {
-    extern __shared__ float sm[];
-    float* S = sm;                 // [dim][64]
-    float* ns = sm + dim * 64;     // [dim]
-    float* ks = ns + dim;          // [dim]
-    float* qs = ks + dim;          // [dim]
-    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x, c = blockIdx.z * 64 + lane;
+// Every thread of wave w carries the same copy of its wave's n values and of m; value tile 0 writes them back.
+template <int DPW>
+__global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_mlstm_scan(const float* proj, long ldp, float* out, long ldo, float* state,
+                                                                          const int* req_rows, const int* req_state, const int* pos, int H,
+                                                                          int dim, int vdim, float cap) {
+    __shared__ float ks[HB_SCAN_MAX_WAVES * DPW], qs[HB_SCAN_MAX_WAVES * DPW], part[HB_SCAN_MAX_WAVES][64], npart[HB_SCAN_MAX_WAVES];
+    const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.z * 64 + lane;
+    const int nw = blockDim.x >> 6, d0 = w * DPW;
     const int rs = req_rows[r], re = req_rows[r + 1];
     if (rs >= re) return;
     const bool ok = c < vdim, fresh = pos[rs] == 0;
     const size_t per = (size_t)dim * vdim + dim + 1;
     float* St = state + ((size_t)req_state[r] * H + h) * per;
     float* nt = St + (size_t)dim * vdim;
-    for (int d = 0; d < dim; ++d) S[d * 64 + lane] = (ok && !fresh) ? St[(size_t)d * vdim + c] : 0.f;
-    for (int d = lane; d < dim; d += 64) ns[d] = fresh ? 0.f : nt[d];
+    float S[DPW], nn[DPW];
+#pragma unroll
+    for (int i = 0; i < DPW; ++i) {
+        S[i] = (ok && !fresh && d0 + i < dim) ? St[(size_t)(d0 + i) * vdim + c] : 0.f;
+        nn[i] = (!fresh && d0 + i < dim) ? nt[d0 + i] : 0.f;
+    }
     float m = fresh ? 0.f : nt[dim];
     const float qscale = 1.0f / sqrtf((float)dim);
     const int off_k = H * dim, off_v = 2 * H * dim, off_i = 2 * H * dim + 2 * H * vdim, off_f = off_i + H;
-    __syncthreads();
     for (int t = rs; t < re; ++t) {
         const float* p = proj + (size_t)t * ldp;
+        for (int d = threadIdx.x; d < nw * DPW; d += blockDim.x) {
+            ks[d] = d < dim ? p[off_k + h * dim + d] : 0.f;
+            qs[d] = d < dim ? p[h * dim + d] * qscale : 0.f;
+        }
         const float ig = cap * tanhf(p[off_i + h] / cap);
         const float fg = hb_logsigmoid(cap * tanhf(p[off_f + h] / cap));
         const float mn = fmaxf(fg + m, ig);
         const float a = expf(fg + m - mn), b = expf(ig - mn);
-        float part = 0.f;
-        for (int d = lane; d < dim; d += 64) {
-            const float kv = p[off_k + h * dim + d], qv = p[h * dim + d] * qscale;
-            const float nn = a * ns[d] + b * kv;
-            ns[d] = nn;
-            ks[d] = kv;
-            qs[d] = qv;
-            part = fmaf(nn, qv, part);
-        }
-        const float nq = hb_wave_sum(part);
-        __syncthreads();
         const float v = ok ? p[off_v + h * vdim + c] : 0.f;
         const float bv = b * v;
-        float o = 0.f;
-        for (int d = 0; d < dim; ++d) {
-            const float s = a * S[d * 64 + lane] + ks[d] * bv;
-            S[d * 64 + lane] = s;
-            o = fmaf(s, qs[d], o);
-        }
-        m = mn;
-        const float den = fmaxf(fabsf(nq), expf(-m)) + 1e-6f;
-        if (ok) out[(size_t)t * ldo + h * vdim + c] = o / den;
         __syncthreads();
+        float o = 0.f, nq = 0.f;
+#pragma unroll
+        for (int i = 0; i < DPW; ++i) {
+            const float kv = ks[d0 + i], qv = qs[d0 + i];
+            nn[i] = a * nn[i] + b * kv;
+            nq = fmaf(nn[i], qv, nq);
+            const float sv = a * S[i] + kv * bv;
+            S[i] = sv;
+            o = fmaf(sv, qv, o);
+        }
+        part[w][lane] = o;
+        if (lane == 0) npart[w] = nq;
+        m = mn;
+        __syncthreads();
+        if (w == 0 && ok) {
+            float sum = part[0][lane], nsum = npart[0];
+            for (int k = 1; k < nw; ++k) { sum += part[k][lane]; nsum += npart[k]; }
+            out[(size_t)t * ldo + h * vdim + c] = sum / (fmaxf(fabsf(nsum), expf(-m)) + 1e-6f);
+        }
     }
-    if (ok)
-        for (int d = 0; d < dim; ++d) St[(size_t)d * vdim + c] = S[d * 64 + lane];
-    if (blockIdx.z == 0) {
-        for (int d = lane; d < dim; d += 64) nt[d] = ns[d];
-        if (lane == 0) nt[dim] = m;
-    }
+#pragma unroll
+    for (int i = 0; i < DPW; ++i)
+        if (d0 + i < dim) {
+            if (ok) St[(size_t)(d0 + i) * vdim + c] = S[i];
+            if (blockIdx.z == 0 && lane == 0) nt[d0 + i] = nn[i];
+        }
+    if (blockIdx.z == 0 && threadIdx.x == 0) nt[dim] = m;
 }
 
 // per (row, head): o / rms(o) over vdim, times a weight (per_head_w: indexed over all heads, else shared [vdim]), times
@@ -513,85 +556,162 @@ __global__ __launch_bounds__(64) void k_hb_pool_update(const T* cache, float* po
     }
 }
 
-// One block per (row, kv head); one wave per query head of the group.  Keys of a row at position p: the pooled blocks
-// 0 .. nb-1 (nb = floor((p - window + 1) / P), those wholly before the window) and then the tokens max(0, p-window+1) .. p.
-// 64 keys at a time: lane = key (score), then lane = value column; running maximum / sum across the chunks in ascending order.
+// One block per (row, kv head).  Keys of a row at position p: the pooled blocks 0 .. nb-1 (nb = floor((p - window + 1) / P), those
+// wholly before the window) and then the tokens max(0, p-window+1) .. p.  The block has SPLIT waves per query head of the group; wave
+// (head, s) takes the 64-key chunks s, s + SPLIT, ... in ascending order: lane = key for the scores, lane = value column for the
+// weighted sum, running maximum and sum across its chunks; the SPLIT partial results of a head are merged in split order.  SPLIT is a
+// property of the layer (its group size), so a row's arithmetic does not depend on the step it is part of.
 #define HB_MAX_VPL 8   // value columns per lane: vdim <= 512
+__device__ __forceinline__ float hb_dot_row(const float* q, const float* k, int dim, bool vec) {
+    float dot = 0.f;
+    if (vec) {
+        for (int d = 0; d < dim; d += 4) {
+            const float4 a = *(const float4*)(q + d), b = *(const float4*)(k + d);
+            dot = fmaf(a.x, b.x, dot); dot = fmaf(a.y, b.y, dot); dot = fmaf(a.z, b.z, dot); dot = fmaf(a.w, b.w, dot);
+        }
+    } else {
+        for (int d = 0; d < dim; ++d) dot = fmaf(q[d], k[d], dot);
+    }
+    return dot;
+}
+__device__ __forceinline__ float hb_dot_row(const float* q, const bf16_t* k, int dim, bool vec) {
+    float dot = 0.f;
+    if (vec) {
+        for (int d = 0; d < dim; d += 8) {
+            const uint4 u = *(const uint4*)(k + d);
+            const float4 a = *(const float4*)(q + d), b = *(const float4*)(q + d + 4);
+            dot = fmaf(a.x, bflo(u.x), dot); dot = fmaf(a.y, bfhi(u.x), dot); dot = fmaf(a.z, bflo(u.y), dot); dot = fmaf(a.w, bfhi(u.y), dot);
+            dot = fmaf(b.x, bflo(u.z), dot); dot = fmaf(b.y, bfhi(u.z), dot); dot = fmaf(b.z, bflo(u.w), dot); dot = fmaf(b.w, bfhi(u.w), dot);
+        }
+    } else {
+        for (int d = 0; d < dim; ++d) dot = fmaf(q[d], bf2f(k[d]), dot);
+    }
+    return dot;
+}
 template <typename T>
 __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
                           const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
-                          long v_base, float scale) {
+                          long v_base, float scale, int split) {
     extern __shared__ float sm[];
-    const int QG = H / G;
-    long* loc = (long*)sm;                 // [QG][64]  (>= 0: token index in the cache, < 0: -(pool entry) - 1)
-    float* pr = sm + QG * 128;             // [QG][64]
-    float* qs = pr + QG * 64;              // [QG][dim]
+    const int QG = H / G, NWV = QG * split;
+    const int dimp = (dim + 3) & ~3;
+    long* loc = (long*)sm;                  // [NWV][64]  (>= 0: token index in the cache, < 0: -(pool entry) - 1)
+    float* pr = sm + NWV * 128;             // [NWV][64]
+    float* qs = pr + NWV * 64;              // [QG][dimp]
+    float* mo = qs + QG * dimp;             // [NWV][vdim + 2]: partial output, maximum, sum of each wave
     const int row = blockIdx.x, g = blockIdx.y, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
-    const int hq = g * QG + wv;
+    const int qh = wv % QG, sp = wv / QG, hq = g * QG + qh;
     const int p = pos[row];
     const int* pt = ptab + (size_t)row_req[row] * pts;
     const int first = p - window + 1;
     const int lo = first > 0 ? first : 0;
     const int nb = first > 0 ? first / P : 0;
     const int total = nb + (p - lo + 1);
-    const float* q = proj + (size_t)row * ldp + hq * dim;
-    for (int d = lane; d < dim; d += 64) qs[wv * dim + d] = q[d];
+    for (int i = threadIdx.x; i < QG * dimp; i += blockDim.x) {
+        const int hh = i / dimp, d = i % dimp;
+        qs[i] = d < dim ? proj[(size_t)row * ldp + (g * QG + hh) * dim + d] : 0.f;
+    }
     __syncthreads();
+    const float* q = qs + qh * dimp;
+    const int pw = dim + vdim;
+    const bool kvec = (dim % (sizeof(T) == 2 ? 8 : 4)) == 0, pvec = (dim % 4 == 0) && (pw % 4 == 0);
     float m = -INFINITY, l = 0.f, acc[HB_MAX_VPL];
 #pragma unroll
     for (int e = 0; e < HB_MAX_VPL; ++e) acc[e] = 0.f;
-    const int pw = dim + vdim;
-    for (int base = 0; base < total; base += 64) {
+    long* wloc = loc + wv * 64;
+    float* wpr = pr + wv * 64;
+    for (int base = sp * 64; base < total; base += split * 64) {
         const int u = base + lane;
-        float s = -INFINITY;
+        float sc = -INFINITY;
         long where = 0;
         if (u < total) {
-            float dot = 0.f;
+            float dot;
             if (u < nb) {
                 const int t = u * P + P - 1;
                 const size_t entry = ((size_t)pt[t / ps] * ppp + (t % ps) / P) * G + g;
-                const float* kp = pool + entry * pw;
-                for (int d = 0; d < dim; ++d) dot = fmaf(qs[wv * dim + d], kp[d], dot);
+                dot = hb_dot_row(q, pool + entry * pw, dim, pvec);
                 where = -(long)entry - 1;
             } else {
                 const int j = lo + (u - nb);
                 const size_t tok = (size_t)pt[j / ps] * ps + j % ps;
-                const T* kp = cache + tok * (size_t)(G * dim) + g * dim;
-                for (int d = 0; d < dim; ++d) dot = fmaf(qs[wv * dim + d], hb_ld(kp + d), dot);
+                dot = hb_dot_row(q, cache + tok * (size_t)(G * dim) + g * dim, dim, kvec);
                 where = (long)tok;
             }
-            s = dot * scale;
+            sc = dot * scale;
         }
-        const float mn = fmaxf(m, hb_wave_max(s));
+        const float mn = fmaxf(m, hb_wave_max(sc));
         const float alpha = expf(m - mn);
-        const float e = u < total ? expf(s - mn) : 0.f;
+        const float e = u < total ? expf(sc - mn) : 0.f;
         l = l * alpha + hb_wave_sum(e);
         m = mn;
-        pr[wv * 64 + lane] = e;
-        loc[wv * 64 + lane] = where;
-        __syncthreads();
+        __builtin_amdgcn_wave_barrier();
+        wpr[lane] = e;
+        wloc[lane] = where;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
         const int cnt = total - base < 64 ? total - base : 64;
+        // pooled keys come first in the key order: two loops without a per-key branch, eight independent requests in flight each
+        const int npool = nb - base < 0 ? 0 : (nb - base < cnt ? nb - base : cnt);
+        const size_t gv = (size_t)G * vdim;
 #pragma unroll
         for (int c = 0; c < HB_MAX_VPL; ++c) {
             const int j = lane + c * 64;
-            if (j < vdim) {
+            if (c * 64 < vdim) {
+                const int jj = j < vdim ? j : vdim - 1;
+                const float* pbase = pool + dim + jj;
+                const T* vbase = cache + v_base + g * vdim + jj;
                 float a = acc[c] * alpha;
-                for (int kk = 0; kk < cnt; ++kk) {
-                    const long w = loc[wv * 64 + kk];
-                    const float vv = w < 0 ? pool[(size_t)(-w - 1) * pw + dim + j]
-                                           : hb_ld(cache + v_base + (size_t)w * (size_t)(G * vdim) + g * vdim + j);
-                    a = fmaf(pr[wv * 64 + kk], vv, a);
+                for (int k0 = 0; k0 < npool; k0 += 8) {
+                    float pv[8], vv[8];
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) {
+                        const int kk = k0 + x < npool ? k0 + x : npool - 1;
+                        pv[x] = k0 + x < npool ? wpr[kk] : 0.f;
+                        vv[x] = pbase[(size_t)(-wloc[kk] - 1) * pw];
+                    }
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) a = fmaf(pv[x], vv[x], a);
+                }
+                for (int k0 = npool; k0 < cnt; k0 += 8) {
+                    float pv[8], vv[8];
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) {
+                        const int kk = k0 + x < cnt ? k0 + x : cnt - 1;
+                        pv[x] = k0 + x < cnt ? wpr[kk] : 0.f;
+                        vv[x] = hb_ld(vbase + (size_t)wloc[kk] * gv);
+                    }
+#pragma unroll
+                    for (int x = 0; x < 8; ++x) a = fmaf(pv[x], vv[x], a);
                 }
                 acc[c] = a;
             }
         }
-        __syncthreads();
+        __builtin_amdgcn_wave_barrier();
     }
-    const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
+    // merge the splits of each head in split order
+    float* mine = mo + (size_t)wv * (vdim + 2);
 #pragma unroll
-    for (int c = 0; c < HB_MAX_VPL; ++c) {
-        const int j = lane + c * 64;
-        if (j < vdim) out[(size_t)row * ldo + hq * vdim + j] = acc[c] / l * gate;
+    for (int c = 0; c < HB_MAX_VPL; ++c)
+        if (lane + c * 64 < vdim) mine[lane + c * 64] = acc[c];
+    if (lane == 0) { mine[vdim] = m; mine[vdim + 1] = l; }
+    __syncthreads();
+    if (sp == 0) {
+        float mm = -INFINITY;
+        for (int s2 = 0; s2 < split; ++s2) mm = fmaxf(mm, mo[(size_t)(s2 * QG + qh) * (vdim + 2) + vdim]);
+        float lt = 0.f;
+        for (int s2 = 0; s2 < split; ++s2) {
+            const float* o2 = mo + (size_t)(s2 * QG + qh) * (vdim + 2);
+            lt += o2[vdim + 1] * expf(o2[vdim] - mm);
+        }
+        const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
+        for (int j = lane; j < vdim; j += 64) {
+            float a = 0.f;
+            for (int s2 = 0; s2 < split; ++s2) {
+                const float* o2 = mo + (size_t)(s2 * QG + qh) * (vdim + 2);
+                a += o2[j] * expf(o2[vdim] - mm);
+            }
+            out[(size_t)row * ldo + hq * vdim + j] = a / lt * gate;
+        }
     }
 }
 
@@ -602,6 +722,32 @@ __global__ void k_hb_copy_rows(const float* src, long lds_, float* dst, long ldd
 __global__ void k_hb_logits_bf16(const float* src, bf16_t* dst, long n) {
     const long i = (long)blockIdx.x * 256 + threadIdx.x;
     if (i < n) dst[i] = f2bf(src[i]);
+}
+// greedy pick on the fp32 logits: first maximum of each row
+__global__ __launch_bounds__(1024) void k_hb_argmax(const float* logits, int V, int* out_ids) {
+    __shared__ float bv[16];
+    __shared__ int bi[16];
+    const int row = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const float* p = logits + (size_t)row * V;
+    float best = -INFINITY;
+    int at = 0x7fffffff;
+    for (int i = threadIdx.x; i < V; i += 1024) {
+        const float v = p[i];
+        if (v > best || (v == best && i < at)) { best = v; at = i; }
+    }
+#pragma unroll
+    for (int o = 32; o >= 1; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64);
+        const int oi = __shfl_xor(at, o, 64);
+        if (ov > best || (ov == best && oi < at)) { best = ov; at = oi; }
+    }
+    if (lane == 0) { bv[wv] = best; bi[wv] = at; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w)
+            if (bv[w] > best || (bv[w] == best && bi[w] < at)) { best = bv[w]; at = bi[w]; }
+        out_ids[row] = at == 0x7fffffff ? 0 : at;
+    }
 }
 __global__ void k_hb_feedback(const int* out_ids, int* input_ids, uint64_t* rng, int B, int feedback) {
     const int b = blockIdx.x * blockDim.x + threadIdx.x;
@@ -649,15 +795,18 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
         hipLaunchKernelGGL(k_hb_layernorm, dim3(n), dim3(256), 0, st, cur, ldx, (const int*)nullptr, L.norm1, m->h, (long)W, W, c.eps);
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->h, W, (const T*)L.w_in, L.b_in, m->proj, n_in, n, n_in, W));
         const int vt = (L.vdim + 63) / 64;
+        // dims per wave of the scans: the smallest of 16 / 32 / 64 that covers dim with at most 16 waves
+        const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
+        const int nwv = (L.dim + dpw - 1) / dpw;
         if (L.kind == VOX_MIXER_HGRN2) {
-            const size_t lds = (size_t)(L.dim * 64 + 2 * L.dim) * 4;
-            hipLaunchKernelGGL(k_hb_hgrn2_scan, dim3(n_req, L.heads, vt), dim3(64), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, L.lower,
+            auto kern = dpw == 16 ? k_hb_hgrn2_scan<16> : (dpw == 32 ? k_hb_hgrn2_scan<32> : k_hb_hgrn2_scan<64>);
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), 0, st, m->proj, (long)n_in, m->mix, (long)n_mix, L.lower,
                                run.state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim);
             hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 0, m->proj, (long)n_in, -1,
                                L.vdim, c.eps);
         } else if (L.kind == VOX_MIXER_MLSTM) {
-            const size_t lds = (size_t)(L.dim * 64 + 3 * L.dim) * 4;
-            hipLaunchKernelGGL(k_hb_mlstm_scan, dim3(n_req, L.heads, vt), dim3(64), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, run.state,
+            auto kern = dpw == 16 ? k_hb_mlstm_scan<16> : (dpw == 32 ? k_hb_mlstm_scan<32> : k_hb_mlstm_scan<64>);
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), 0, st, m->proj, (long)n_in, m->mix, (long)n_mix, run.state,
                                io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap);
             hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_in,
                                2 * L.heads * L.dim + L.heads * L.vdim, L.vdim, c.eps);
@@ -669,10 +818,12 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
                                io->page, io->slot, H, G, L.dim, L.vdim, L.rot_dims, ps, v_base, c.eps);
             hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)run.cache, run.pool, io->pos, io->row_req,
                                io->page_table, io->pt_stride, G, L.dim, L.vdim, L.pool, ps, ppp, v_base);
-            const size_t lds = (size_t)QG * L.dim * 4 + (size_t)QG * 64 * 4 + (size_t)QG * 64 * 8;
-            hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G), dim3(64 * QG), lds, st, m->proj, (long)n_in, (const T*)run.cache, run.pool, m->mix,
+            const int split = QG >= 8 ? 1 : (QG >= 4 ? 2 : 4);
+            const int nwv2 = QG * split, dimp = (L.dim + 3) & ~3;
+            const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (L.vdim + 2) * 4;
+            hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G), dim3(64 * nwv2), lds, st, m->proj, (long)n_in, (const T*)run.cache, run.pool, m->mix,
                                (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, L.window, L.pool, ps, ppp,
-                               v_base, L.scale);
+                               v_base, L.scale, split);
         }
         VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix));
         if (L.ff > 0) {
@@ -713,7 +864,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         else if (L.ff > 0 && (!L.norm2 || !L.w_up || !L.w_down)) bad = "missing feed-forward weights";
         else if (L.kind == VOX_MIXER_HGRN2 && (!L.lower || !L.head_norm)) bad = "hgrn2 needs lower and head_norm";
         else if (L.kind == VOX_MIXER_MLSTM && (!L.head_norm || !(L.gate_cap > 0.f))) bad = "mlstm needs head_norm and gate_cap";
-        else if (L.kind != VOX_MIXER_POOLED_WINDOW_ATTN && (size_t)(L.dim * 64 + 3 * L.dim) * 4 > 160 * 1024) bad = "dim too large for the LDS state tile";
+        else if (L.kind != VOX_MIXER_POOLED_WINDOW_ATTN && L.dim > 64 * HB_SCAN_MAX_WAVES) bad = "recurrent dim above 1024";
         else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN) {
             if (L.kv_heads < 1 || L.heads % L.kv_heads != 0 || L.heads / L.kv_heads > 16) bad = "heads / kv_heads (group of at most 16)";
             else if (L.dim > 64 * HB_MAX_DPL) bad = "dim above 512";
@@ -764,6 +915,14 @@ int vox_hybrid_step(vox_hybrid* m, void* stream, const vox_hybrid_io* io, const 
     if (!sc) return VOX_OK;
     // sampling: one pick per request from the first n_req output rows (the caller lists each request's last row first)
     if (n_out < n_req || n_req > c.max_batch || !io->out_ids) return vox_fail(VOX_ERR_INVALID, "hybrid_step: sampling needs one output row per request");
+    if (sc->greedy) {
+        hipLaunchKernelGGL(k_hb_argmax, dim3(n_req), dim3(1024), 0, st, io->logits, c.vocab, io->out_ids);
+        if (feedback || io->rng_offset)
+            hipLaunchKernelGGL(k_hb_feedback, dim3((n_req + 63) / 64), dim3(64), 0, st, io->out_ids, io->input_ids, io->rng_offset, n_req,
+                               feedback && io->input_ids ? 1 : 0);
+        return VOX_OK;
+    }
+    // stochastic modes: the library's sampler (bf16 logits, Philox stream keyed by seed and the engine's step counter)
     const long nl = (long)n_req * c.vocab;
     hipLaunchKernelGGL(k_hb_logits_bf16, dim3((unsigned)((nl + 255) / 256)), dim3(256), 0, st, io->logits, m->logits16, nl);
     SampleCall s;

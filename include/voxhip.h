@@ -389,7 +389,7 @@ typedef struct {
     float* state;        /* HGRN2: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1] */
 } vox_hybrid_run;
 typedef struct {
-    int32_t width, vocab, n_layers, n_runs, dtype, page_size, max_rows, max_batch, max_out, max_pages;
+    int32_t width, vocab, n_layers, n_runs, dtype, page_size, max_rows, max_batch, max_out, max_pages, max_seq_len;
     float eps;
 } vox_hybrid_config;
 typedef struct {
@@ -412,9 +412,10 @@ typedef struct {
 } vox_hybrid_io;
 int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybrid_weights* w, vox_hybrid** out);
 void vox_hybrid_destroy(vox_hybrid* m);
-/* ids: [n_rows] token ids of the rows.  sampling NULL: logits only; else one pick per request from output rows 0..n_req-1. */
+/* ids: [n_rows] token ids of the rows.  max_kvlen: a bound on (position + 1) of every row (grid bound of the attention; 0 = the
+ * engine's max_seq_len).  sampling NULL: logits only; else one pick per request from output rows 0..n_req-1. */
 int vox_hybrid_step(vox_hybrid* m, void* stream, const vox_hybrid_io* io, const int32_t* ids, int n_rows, int n_req, int n_out,
-                    const vox_sampling_config* sampling, uint64_t seed, int feedback);
+                    int max_kvlen, const vox_sampling_config* sampling, uint64_t seed, int feedback);
 
 /* ---- Qwen3-TTS 12 Hz codec decoder (token -> waveform), streaming ------------------------------------
  * replaces Qwen3TTSTokenizerV2Decoder.forward_chunk (tokenizer/qwen3_codec.py:1541-1666), the DecoderCache

@@ -28,14 +28,14 @@ def tokens(n, vocab, seed):
     return torch.randint(0, vocab, (n,), generator=torch.Generator().manual_seed(seed)).tolist()
 
 
-def check(cfg, S, toks, cuts, dtype=torch.float32, bar=None, **kw):
+def check(cfg, S, toks, cuts, dtype=torch.float32, bar=None, quantile=None, **kw):
     want = HR.forward(cfg, S, toks)
     d = U.Driver(cfg, S, dtype=dtype, **kw)
     try:
         got = d.run_cut("r", toks, cuts)
     finally:
         d.close()
-    err = U.rel_err(got, want)
+    err = U.rel_err(got, want, quantile)
     assert err < (bar or (F32_BAR if dtype == torch.float32 else BF16_BAR)), err
     return got
 
@@ -210,6 +210,19 @@ def test_pool_blocks_across_page_borders(page_size, pool):
     S = U.random_checkpoint(cfg, seed=27, gain=2.0)
     toks = tokens(90, 32, 28)
     check(cfg, S, toks, [11, 2, 29], page_size=page_size, pages=32)
+
+
+def test_many_keys_few_rows():
+    """More than 256 visible keys (window 150 + up to 135 pooled blocks of 2): steps of few rows split the keys over several
+    blocks and merge; prompts of many rows do not.  Both against the same oracle, sharp softmax."""
+    toks = tokens(420, 40, 42)
+    for scale, dtype, q in ((2.0, torch.float32, None), (None, torch.bfloat16, 0.9)):
+        cfg = U.config([U.attention(heads=4, kv_heads=2, dim=16, vdim=24, window=150, pool=2, rot=8, scale=scale), U.mlstm()], width=24, vocab=40)
+        S = U.random_checkpoint(cfg, seed=41)
+        # (bf16: the mLSTM's normaliser max(|n.q|, exp(-m)) amplifies rounding at a few positions, in every schedule alike: 90 % bar)
+        a = check(cfg, S, toks, [420], pages=64, max_rows=512, dtype=dtype, quantile=q)
+        b = check(cfg, S, toks, [330, 3, 2, 20], pages=64, max_rows=512, dtype=dtype, quantile=q)   # 20-, 3- and 1-row steps over 280+ keys
+        assert U.rel_err(b, a.double(), 0.9) < (F32_BAR if dtype == torch.float32 else BF16_BAR)
 
 
 def test_long_decoding():

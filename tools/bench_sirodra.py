@@ -68,7 +68,7 @@ def bench_hybrid(width, blocks, vocab, prompts, batches, ctx, steps, warmup, dev
         npg = (n + ps - 1) // ps
         eng.upload_plan(pos=np.arange(n), kvlen=np.arange(1, n + 1), page=np.arange(n) // ps, slot=np.arange(n) % ps, q_req=np.zeros(n),
                         last_rows=[n - 1], indptr=[0, npg], indices=np.arange(npg), req_rows=[0, n], state=[0])
-        dt = time_steps(lambda: eng.step(n, 1, 1, sc, feedback=False), max(3, steps // 5), 2)
+        dt = time_steps(lambda: eng.step(n, 1, 1, sc, feedback=False, max_kvlen=n), max(3, steps // 5), 2)
         out["prefill"][str(n)] = {"ms": dt * 1e3, "tokens_per_s": n / dt}
     for B in batches:
         # every request has `ctx` tokens behind it (cache contents are whatever the pages hold: timing only)

@@ -241,8 +241,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
 
 // 1..8 rows (decode): a wave streams CPW weight rows (output columns) at once, 16 bytes per lane and request, against one read of
 // the activations; lanes own k-chunks c, c + 64, ...; butterfly at the end.  The order of each output's sum depends on K only.
-#define HB_GEMV_CPW 4
-template <typename T, int MR, int EPI>
+template <typename T, int MR, int EPI, int HB_GEMV_CPW>
 __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const T* Wt, const float* bias, float* C, long ldc, int M, int N,
                                                  int K) {
     const int lane = threadIdx.x & 63, n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * HB_GEMV_CPW;
@@ -327,11 +326,19 @@ int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const float* W, cons
 template <typename T, int EPI>
 int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
     if (M <= 0 || N <= 0) return VOX_OK;
-    const dim3 g((N + 4 * HB_GEMV_CPW - 1) / (4 * HB_GEMV_CPW)), b(256);
-    if (M == 1) hipLaunchKernelGGL((k_hb_gemv<T, 1, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
-    else if (M == 2) hipLaunchKernelGGL((k_hb_gemv<T, 2, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
-    else if (M <= 4) hipLaunchKernelGGL((k_hb_gemv<T, 4, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
-    else if (M <= 8) hipLaunchKernelGGL((k_hb_gemv<T, 8, EPI>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    // four columns per wave once that still leaves a block for every compute unit several times over
+    const bool wide = N >= 16 * 1024;
+    const dim3 g(wide ? (N + 15) / 16 : (N + 3) / 4), b(256);
+#define HB_GEMV(MR_) \
+    do { \
+        if (wide) hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 4>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K); \
+        else hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 1>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K); \
+    } while (0)
+    if (M == 1) HB_GEMV(1);
+    else if (M == 2) HB_GEMV(2);
+    else if (M <= 4) HB_GEMV(4);
+    else if (M <= 8) HB_GEMV(8);
+#undef HB_GEMV
     else return hb_gemm_tiles<EPI>(st, A, lda, W, bias, C, ldc, M, N, K);
     return VOX_OK;
 }
@@ -562,6 +569,8 @@ __global__ __launch_bounds__(64) void k_hb_pool_update(const T* cache, float* po
 // weighted sum, running maximum and sum across its chunks; the SPLIT partial results of a head are merged in split order.  SPLIT is a
 // property of the layer (its group size), so a row's arithmetic does not depend on the step it is part of.
 #define HB_MAX_VPL 8   // value columns per lane: vdim <= 512
+#define HB_ATTN_SEG 4        // 64-key chunks per block of a segmented launch
+#define HB_ATTN_SEG_ROWS 32  // steps of at most this many rows are segmented
 __device__ __forceinline__ float hb_dot_row(const float* q, const float* k, int dim, bool vec) {
     float dot = 0.f;
     if (vec) {
@@ -591,7 +600,7 @@ __device__ __forceinline__ float hb_dot_row(const float* q, const bf16_t* k, int
 template <typename T>
 __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
                           const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
-                          long v_base, float scale, int split) {
+                          long v_base, float scale, int split, int seg_chunks, float* part) {
     extern __shared__ float sm[];
     const int QG = H / G, NWV = QG * split;
     const int dimp = (dim + 3) & ~3;
@@ -607,6 +616,11 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
     const int lo = first > 0 ? first : 0;
     const int nb = first > 0 ? first / P : 0;
     const int total = nb + (p - lo + 1);
+    // few-row steps: block z takes the chunks [z * seg_chunks, (z + 1) * seg_chunks) and leaves an unnormalised partial result
+    const int nchunks = (total + 63) >> 6;
+    const int c0 = seg_chunks > 0 ? blockIdx.z * seg_chunks : 0;
+    const int c1 = seg_chunks > 0 && c0 + seg_chunks < nchunks ? c0 + seg_chunks : nchunks;
+    if (c0 >= nchunks) return;
     for (int i = threadIdx.x; i < QG * dimp; i += blockDim.x) {
         const int hh = i / dimp, d = i % dimp;
         qs[i] = d < dim ? proj[(size_t)row * ldp + (g * QG + hh) * dim + d] : 0.f;
@@ -620,7 +634,7 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
     for (int e = 0; e < HB_MAX_VPL; ++e) acc[e] = 0.f;
     long* wloc = loc + wv * 64;
     float* wpr = pr + wv * 64;
-    for (int base = sp * 64; base < total; base += split * 64) {
+    for (int base = (c0 + sp) * 64; base < c1 * 64; base += split * 64) {
         const int u = base + lane;
         float sc = -INFINITY;
         long where = 0;
@@ -672,16 +686,16 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
 #pragma unroll
                     for (int x = 0; x < 8; ++x) a = fmaf(pv[x], vv[x], a);
                 }
-                for (int k0 = npool; k0 < cnt; k0 += 8) {
-                    float pv[8], vv[8];
+                for (int k0 = npool; k0 < cnt; k0 += 16) {
+                    float pv[16], vv[16];
 #pragma unroll
-                    for (int x = 0; x < 8; ++x) {
+                    for (int x = 0; x < 16; ++x) {
                         const int kk = k0 + x < cnt ? k0 + x : cnt - 1;
                         pv[x] = k0 + x < cnt ? wpr[kk] : 0.f;
                         vv[x] = hb_ld(vbase + (size_t)wloc[kk] * gv);
                     }
 #pragma unroll
-                    for (int x = 0; x < 8; ++x) a = fmaf(pv[x], vv[x], a);
+                    for (int x = 0; x < 16; ++x) a = fmaf(pv[x], vv[x], a);
                 }
                 acc[c] = a;
             }
@@ -703,6 +717,19 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
             const float* o2 = mo + (size_t)(s2 * QG + qh) * (vdim + 2);
             lt += o2[vdim + 1] * expf(o2[vdim] - mm);
         }
+        if (part) {
+            float* dst = part + ((size_t)(row * H + hq) * gridDim.z + blockIdx.z) * (vdim + 2);
+            for (int j = lane; j < vdim; j += 64) {
+                float a = 0.f;
+                for (int s2 = 0; s2 < split; ++s2) {
+                    const float* o2 = mo + (size_t)(s2 * QG + qh) * (vdim + 2);
+                    a += o2[j] * expf(o2[vdim] - mm);
+                }
+                dst[j] = a;
+            }
+            if (lane == 0) { dst[vdim] = mm; dst[vdim + 1] = lt; }
+            return;
+        }
         const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
         for (int j = lane; j < vdim; j += 64) {
             float a = 0.f;
@@ -712,6 +739,27 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
             }
             out[(size_t)row * ldo + hq * vdim + j] = a / lt * gate;
         }
+    }
+}
+
+// few-row steps: the segments' partial results of a (row, head), merged in segment order; output gate applied here
+__global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nseg_grid, const float* proj, long ldp, float* out, long ldo,
+                                                      const int* pos, int H, int G, int dim, int vdim, int window, int P, int seg_chunks) {
+    const int row = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
+    const int p = pos[row];
+    const int first = p - window + 1;
+    const int total = (first > 0 ? first / P : 0) + (p - (first > 0 ? first : 0) + 1);
+    const int nseg = (((total + 63) >> 6) + seg_chunks - 1) / seg_chunks;
+    const float* src = part + (size_t)(row * H + hq) * nseg_grid * (vdim + 2);
+    float mm = -INFINITY;
+    for (int s2 = 0; s2 < nseg; ++s2) mm = fmaxf(mm, src[(size_t)s2 * (vdim + 2) + vdim]);
+    float lt = 0.f;
+    for (int s2 = 0; s2 < nseg; ++s2) lt += src[(size_t)s2 * (vdim + 2) + vdim + 1] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
+    const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
+    for (int j = lane; j < vdim; j += 64) {
+        float a = 0.f;
+        for (int s2 = 0; s2 < nseg; ++s2) a += src[(size_t)s2 * (vdim + 2) + j] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
+        out[(size_t)row * ldo + hq * vdim + j] = a / lt * gate;
     }
 }
 
@@ -765,6 +813,8 @@ struct vox_hybrid {
     vox_hybrid_weights w;
     float *xa = nullptr, *xb = nullptr, *h = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
     bf16_t* logits16 = nullptr;
+    float* attn_ws = nullptr;
+    size_t attn_ws_bytes = 0;
     int max_in = 0, max_mix = 0, max_ff = 0;
 };
 
@@ -778,7 +828,7 @@ static int hb_layer_in(const vox_hybrid_layer& L) {
 }
 
 template <typename T>
-static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const int32_t* ids, int n, int n_req, int n_out) {
+static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const int32_t* ids, int n, int n_req, int n_out, int max_kvlen) {
     const vox_hybrid_config& c = m->cfg;
     const int W = c.width, ps = c.page_size;
     const long ldx = 2L * W;
@@ -821,9 +871,17 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             const int split = QG >= 8 ? 1 : (QG >= 4 ? 2 : 4);
             const int nwv2 = QG * split, dimp = (L.dim + 3) & ~3;
             const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (L.vdim + 2) * 4;
-            hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G), dim3(64 * nwv2), lds, st, m->proj, (long)n_in, (const T*)run.cache, run.pool, m->mix,
-                               (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, L.window, L.pool, ps, ppp,
-                               v_base, L.scale, split);
+            // steps of few rows: 4-chunk key segments on separate blocks + a merge pass (more blocks than rows x kv heads); a row's
+            // result differs from the one-block form by the rounding of the merge only
+            const int max_keys = (max_kvlen < L.window ? max_kvlen : L.window) + max_kvlen / L.pool + 1;
+            const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
+            const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (L.vdim + 2) * 4 <= m->attn_ws_bytes;
+            hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, m->proj, (long)n_in, (const T*)run.cache,
+                               run.pool, m->mix, (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, L.window,
+                               L.pool, ps, ppp, v_base, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr);
+            if (segmented)
+                hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->proj, (long)n_in, m->mix, (long)n_mix,
+                                   io->pos, H, G, L.dim, L.vdim, L.window, L.pool, HB_ATTN_SEG);
         }
         VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix));
         if (L.ff > 0) {
@@ -847,7 +905,7 @@ extern "C" {
 int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybrid_weights* w, vox_hybrid** out) {
     if (!ctx || !cfg || !w || !out || !w->layers || !w->runs) return vox_fail(VOX_ERR_INVALID, "hybrid_create: NULL argument");
     if (cfg->dtype != VOX_HYBRID_BF16 && cfg->dtype != VOX_HYBRID_F32) return vox_fail(VOX_ERR_INVALID, "hybrid_create: dtype %d", cfg->dtype);
-    if (cfg->width < 1 || cfg->vocab < 1 || cfg->page_size < 1 || cfg->max_rows < 1 || cfg->max_batch < 1 || cfg->max_out < 1)
+    if (cfg->width < 1 || cfg->vocab < 1 || cfg->page_size < 1 || cfg->max_rows < 1 || cfg->max_batch < 1 || cfg->max_out < 1 || cfg->max_seq_len < 1)
         return vox_fail(VOX_ERR_INVALID, "hybrid_create: bad sizes");
     vox_hybrid* m = new vox_hybrid();
     m->ctx = ctx; m->cfg = *cfg; m->w = *w;
@@ -890,6 +948,15 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
               hipMalloc((void**)&m->ff, R * (size_t)(m->max_ff > 0 ? m->max_ff : 1) * 4) == hipSuccess &&
               hipMalloc((void**)&m->hout, (size_t)cfg->max_out * W * 4) == hipSuccess &&
               hipMalloc((void**)&m->logits16, (size_t)cfg->max_batch * cfg->vocab * 2) == hipSuccess;
+    // partial results of segmented attention launches: few rows x heads x segments of the longest sequence
+    for (const vox_hybrid_layer& L : m->layers)
+        if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN) {
+            const int max_keys = (cfg->max_seq_len < L.window ? cfg->max_seq_len : L.window) + cfg->max_seq_len / L.pool + 1;
+            const size_t nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
+            const size_t b = (size_t)HB_ATTN_SEG_ROWS * L.heads * nseg * (L.vdim + 2) * 4;
+            if (b > m->attn_ws_bytes) m->attn_ws_bytes = b;
+        }
+    if (ok && m->attn_ws_bytes) ok = hipMalloc((void**)&m->attn_ws, m->attn_ws_bytes) == hipSuccess;
     if (!ok) { vox_hybrid_destroy(m); return vox_fail(VOX_ERR_NOMEM, "hybrid_create: hipMalloc failed"); }
     *out = m;
     return VOX_OK;
@@ -898,20 +965,21 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
 void vox_hybrid_destroy(vox_hybrid* m) {
     if (!m) return;
     (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->proj); (void)hipFree(m->mix);
-    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16);
+    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws);
     delete m;
 }
 
 int vox_hybrid_step(vox_hybrid* m, void* stream, const vox_hybrid_io* io, const int32_t* ids, int n_rows, int n_req, int n_out,
-                    const vox_sampling_config* sc, uint64_t seed, int feedback) {
+                    int max_kvlen, const vox_sampling_config* sc, uint64_t seed, int feedback) {
     if (!m || !io || !ids) return vox_fail(VOX_ERR_INVALID, "hybrid_step: NULL");
     const vox_hybrid_config& c = m->cfg;
     if (n_rows < 1 || n_rows > c.max_rows || n_req < 1 || n_req > c.max_batch || n_req > n_rows || n_out < 0 || n_out > c.max_out)
         return vox_fail(VOX_ERR_INVALID, "hybrid_step: rows %d / requests %d / outputs %d out of range", n_rows, n_req, n_out);
     if (!io->pos || !io->row_req || !io->page || !io->slot || !io->req_rows || !io->req_state || !io->page_table || (n_out && (!io->out_rows || !io->logits)))
         return vox_fail(VOX_ERR_INVALID, "hybrid_step: missing plan arrays");
+    if (max_kvlen < 1 || max_kvlen > c.max_seq_len) max_kvlen = c.max_seq_len;
     hipStream_t st = (hipStream_t)stream;
-    VOX_TRY(c.dtype == VOX_HYBRID_F32 ? hb_step<float>(m, st, io, ids, n_rows, n_req, n_out) : hb_step<bf16_t>(m, st, io, ids, n_rows, n_req, n_out));
+    VOX_TRY(c.dtype == VOX_HYBRID_F32 ? hb_step<float>(m, st, io, ids, n_rows, n_req, n_out, max_kvlen) : hb_step<bf16_t>(m, st, io, ids, n_rows, n_req, n_out, max_kvlen));
     if (!sc) return VOX_OK;
     // sampling: one pick per request from the first n_req output rows (the caller lists each request's last row first)
     if (n_out < n_req || n_req > c.max_batch || !io->out_ids) return vox_fail(VOX_ERR_INVALID, "hybrid_step: sampling needs one output row per request");

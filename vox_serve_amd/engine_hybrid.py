@@ -82,7 +82,7 @@ class HybridRunC(ctypes.Structure):
 
 class HybridConfigC(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("width", "vocab", "n_layers", "n_runs", "dtype", "page_size", "max_rows",
-                                              "max_batch", "max_out", "max_pages")] + [("eps", ctypes.c_float)]
+                                              "max_batch", "max_out", "max_pages", "max_seq_len")] + [("eps", ctypes.c_float)]
 
 
 class HybridWeightsC(ctypes.Structure):
@@ -122,7 +122,7 @@ class HybridEngine(Qwen3Engine):
         L, vp, ci = self.L, ctypes.c_void_p, ctypes.c_int
         L.vox_hybrid_create.restype, L.vox_hybrid_create.argtypes = ci, [vp, ctypes.POINTER(HybridConfigC), ctypes.POINTER(HybridWeightsC), ctypes.POINTER(vp)]
         L.vox_hybrid_destroy.restype, L.vox_hybrid_destroy.argtypes = None, [vp]
-        L.vox_hybrid_step.restype, L.vox_hybrid_step.argtypes = ci, [vp, vp, ctypes.POINTER(HybridIO), vp, ci, ci, ci, ctypes.POINTER(N.SamplingCfg), ctypes.c_uint64, ci]
+        L.vox_hybrid_step.restype, L.vox_hybrid_step.argtypes = ci, [vp, vp, ctypes.POINTER(HybridIO), vp, ci, ci, ci, ci, ctypes.POINTER(N.SamplingCfg), ctypes.c_uint64, ci]
         dev = self.device
         self._keep = []
 
@@ -169,7 +169,7 @@ class HybridEngine(Qwen3Engine):
                 rarr[j].state = st.data_ptr()
         self.n_runs = len(runs)
         cc = HybridConfigC(W, cfg.vocab, len(cfg.layers), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
-                           max_batch, self.max_out, max_pages, cfg.eps)
+                           max_batch, self.max_out, max_pages, max_seq_len, cfg.eps)
         cw = HybridWeightsC(ctypes.cast(larr, ctypes.POINTER(HybridLayerC)), ctypes.cast(rarr, ctypes.POINTER(HybridRunC)),
                             mat(weights["embedding"]), mat(weights.get("loop_in")), mat(weights["head"]), vec(weights["final_norm"]))
         self._larr, self._rarr = larr, rarr
@@ -216,27 +216,27 @@ class HybridEngine(Qwen3Engine):
         return [self.input_ids, self.rng_offset] + self.states
 
     def _native_frame(self, io, st, batch, bucket, sampling, seed, feedback):
-        N.check(self.L.vox_hybrid_step(self.h, st, ctypes.byref(io), self.input_ids.data_ptr(), batch, batch, batch,
+        N.check(self.L.vox_hybrid_step(self.h, st, ctypes.byref(io), self.input_ids.data_ptr(), batch, batch, batch, int(bucket),
                                        ctypes.byref(sampling), seed, int(feedback)))
 
     def _native_destroy(self):
         self.L.vox_hybrid_destroy(self.h)
 
-    def step(self, n_rows, n_req, n_out=None, sampling=None, seed=0, feedback=True, sample=True):
+    def step(self, n_rows, n_req, n_out=None, sampling=None, seed=0, feedback=True, sample=True, max_kvlen=0):
         """One ragged step, eagerly: rows staged in row_ids + plan arrays.  n_out rows (plan `last_rows`) get logits in
         out_logits[:n_out]; with `sample`, requests 0..n_req-1 are sampled from output rows 0..n_req-1."""
         n_out = n_req if n_out is None else n_out
         io = self._io()
         sc = ctypes.byref(sampling or self.sampling_cfg()) if sample else None
         self._log_launch("prefill", (n_rows, n_req, n_out), n_req)
-        N.check(self.L.vox_hybrid_step(self.h, N.stream(), ctypes.byref(io), self.row_ids.data_ptr(), n_rows, n_req, n_out, sc, seed,
-                                       int(feedback and sample)))
+        N.check(self.L.vox_hybrid_step(self.h, N.stream(), ctypes.byref(io), self.row_ids.data_ptr(), n_rows, n_req, n_out, int(max_kvlen), sc,
+                                       seed, int(feedback and sample)))
 
     def _prefill_on_stream(self, n_rows, n_req, max_kvlen, sampling, seed, feedback):
         if n_req == 0:
             raise N.VoxError("HybridEngine: a step without requests")
         io = self._io()
-        N.check(self.L.vox_hybrid_step(self.h, N.stream(), ctypes.byref(io), self.row_ids.data_ptr(), n_rows, n_req, n_req,
+        N.check(self.L.vox_hybrid_step(self.h, N.stream(), ctypes.byref(io), self.row_ids.data_ptr(), n_rows, n_req, n_req, int(max_kvlen),
                                        ctypes.byref(sampling), seed, int(feedback)))
 
     @staticmethod

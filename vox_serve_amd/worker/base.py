@@ -369,7 +369,8 @@ class ModelWorker:
                       indptr=lm_inputs["paged_kv_indptr"], indices=lm_inputs["paged_kv_indices"], req_rows=qo,
                       state=[int(getattr(r, "state_slot", 0) or 0) for r in requests])
         ended = [i for i, r in enumerate(requests) if r.done_lm_prefill]
-        e.step(n_rows, n_req, n_out=len(out_rows), sampling=self._sampling(), seed=self.seed, feedback=True, sample=bool(ended))
+        e.step(n_rows, n_req, n_out=len(out_rows), sampling=self._sampling(), seed=self.seed, feedback=True, sample=bool(ended),
+               max_kvlen=max(kvlen))
         self.nvtx_range_pop()
         if ended:
             out = e.out_ids[:n_req].cpu().to(torch.long)

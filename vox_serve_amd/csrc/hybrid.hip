@@ -308,6 +308,64 @@ __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const
         }
 }
 
+// 2..16 rows, bf16: one MFMA row tile; a block owns 16 output columns and its four waves take the 32-wide k-steps w, w + 4, ...
+// with both fragments straight from memory (the weight fragment is one 16-byte request per lane, the activation fragment two,
+// converted to bf16 in registers); the four partial tiles are added in wave order.  Needs K % 32 == 0.
+template <int EPI>
+__global__ __launch_bounds__(256) void k_hb_gemm_rows16(const float* A, long lda, const bf16_t* Wt, const float* bias, float* C, long ldc, int M,
+                                                        int N, int K) {
+    __shared__ float red[4][16][17];
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int n0 = blockIdx.x * 16, col = lane & 15, kb = lane >> 4;
+    const int nsteps = K >> 5;
+    hb_f32x4 acc = hb_f32x4{0.f, 0.f, 0.f, 0.f};
+    const bf16_t* wrow = Wt + (size_t)(n0 + col < N ? n0 + col : N - 1) * K + kb * 8;
+    const float* arow = A + (size_t)(col < M ? col : M - 1) * lda + kb * 8;
+    const bool rowok = col < M;
+    constexpr int U = 8;
+    for (int s0 = wv; s0 < nsteps; s0 += 4 * U) {
+        uint4 wf[U];
+        float4 a0[U], a1[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int sidx = s0 + 4 * u;
+            const bool valid = sidx < nsteps;
+            const int k = (valid ? sidx : s0) << 5;
+            wf[u] = *(const uint4*)(wrow + k);
+            a0[u] = *(const float4*)(arow + k);
+            a1[u] = *(const float4*)(arow + k + 4);
+            if (!valid || !rowok) { a0[u] = make_float4(0.f, 0.f, 0.f, 0.f); a1[u] = a0[u]; }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            union { uint4 q; hb_bf16x8 b; } af, bfv;
+            af.q.x = pack_bf2(a0[u].x, a0[u].y); af.q.y = pack_bf2(a0[u].z, a0[u].w);
+            af.q.z = pack_bf2(a1[u].x, a1[u].y); af.q.w = pack_bf2(a1[u].z, a1[u].w);
+            bfv.q = wf[u];
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(af.b, bfv.b, acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) red[wv][kb * 4 + r][col] = acc[r];
+    __syncthreads();
+    if (wv == 0 && n0 + col < N) {
+        const float bz = bias ? bias[n0 + col] : 0.f;
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            const int row = kb * 4 + r;
+            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col], bz);
+        }
+    }
+}
+template <int EPI>
+bool hb_try_rows16(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K) {
+    if (M < 2 || M > 16 || (K & 31) || (lda & 3) || ((size_t)A & 15) || ((size_t)W & 15)) return false;
+    hipLaunchKernelGGL((k_hb_gemm_rows16<EPI>), dim3((N + 15) / 16), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    return true;
+}
+template <int EPI>
+bool hb_try_rows16(hipStream_t, const float*, long, const float*, const float*, float*, long, int, int, int) { return false; }
+
 template <typename T, int EPI>
 int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K);
 
@@ -334,7 +392,8 @@ int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const floa
         if (wide) hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 4>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K); \
         else hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 1>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K); \
     } while (0)
-    if (M == 1) HB_GEMV(1);
+    if (hb_try_rows16<EPI>(st, A, lda, W, bias, C, ldc, M, N, K)) {}
+    else if (M == 1) HB_GEMV(1);
     else if (M == 2) HB_GEMV(2);
     else if (M <= 4) HB_GEMV(4);
     else if (M <= 8) HB_GEMV(8);
@@ -686,16 +745,16 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
 #pragma unroll
                     for (int x = 0; x < 8; ++x) a = fmaf(pv[x], vv[x], a);
                 }
-                for (int k0 = npool; k0 < cnt; k0 += 16) {
-                    float pv[16], vv[16];
+                for (int k0 = npool; k0 < cnt; k0 += 32) {
+                    float pv[32], vv[32];
 #pragma unroll
-                    for (int x = 0; x < 16; ++x) {
+                    for (int x = 0; x < 32; ++x) {
                         const int kk = k0 + x < cnt ? k0 + x : cnt - 1;
                         pv[x] = k0 + x < cnt ? wpr[kk] : 0.f;
                         vv[x] = hb_ld(vbase + (size_t)wloc[kk] * gv);
                     }
 #pragma unroll
-                    for (int x = 0; x < 16; ++x) a = fmaf(pv[x], vv[x], a);
+                    for (int x = 0; x < 32; ++x) a = fmaf(pv[x], vv[x], a);
                 }
                 acc[c] = a;
             }

@@ -129,8 +129,13 @@ def lib():
         # (seen with `python __graft_entry__.py smoke`, whose build() step loaded the library before anything imported torch)
         import torch  # noqa: F401
         L = ctypes.CDLL(LIB_PATH)
+        reduced = os.path.basename(LIB_PATH) != "libvoxhip.so"
         for name, (res, args) in {**_SIGS, **_OPTIONAL_SIGS}.items():
-            fn = getattr(L, name)
+            # a reduced library (VOX_LIB: one engine's sources only) lacks the other engines' entry points: those stay unbound
+            # and raise on first use; the full library must export every one of them
+            fn = getattr(L, name, None) if reduced else getattr(L, name)
+            if fn is None:
+                continue
             fn.restype, fn.argtypes = res, args
         if L.vox_abi_version() != 1:
             raise VoxError("libvoxhip ABI version mismatch")

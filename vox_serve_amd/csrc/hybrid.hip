@@ -656,8 +656,29 @@ __device__ __forceinline__ float hb_dot_row(const float* q, const bf16_t* k, int
     }
     return dot;
 }
+// one lane's share of a key row under the sixteen-lanes-per-key split: dims [sub*8, sub*8+8) of every 128
+__device__ __forceinline__ float hb_dot_slices(const float* q, const float* k, int dim, int sub) {
+    float part = 0.f;
+    for (int d = sub * 8; d < dim; d += 128) {
+        const float4 k0 = *(const float4*)(k + d), k1 = *(const float4*)(k + d + 4);
+        const float4 a = *(const float4*)(q + d), b = *(const float4*)(q + d + 4);
+        part = fmaf(a.x, k0.x, part); part = fmaf(a.y, k0.y, part); part = fmaf(a.z, k0.z, part); part = fmaf(a.w, k0.w, part);
+        part = fmaf(b.x, k1.x, part); part = fmaf(b.y, k1.y, part); part = fmaf(b.z, k1.z, part); part = fmaf(b.w, k1.w, part);
+    }
+    return part;
+}
+__device__ __forceinline__ float hb_dot_slices(const float* q, const bf16_t* k, int dim, int sub) {
+    float part = 0.f;
+    for (int d = sub * 8; d < dim; d += 128) {
+        const uint4 u = *(const uint4*)(k + d);
+        const float4 a = *(const float4*)(q + d), b = *(const float4*)(q + d + 4);
+        part = fmaf(a.x, bflo(u.x), part); part = fmaf(a.y, bfhi(u.x), part); part = fmaf(a.z, bflo(u.y), part); part = fmaf(a.w, bfhi(u.y), part);
+        part = fmaf(b.x, bflo(u.z), part); part = fmaf(b.y, bfhi(u.z), part); part = fmaf(b.z, bflo(u.w), part); part = fmaf(b.w, bfhi(u.w), part);
+    }
+    return part;
+}
 template <typename T>
-__global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
+__global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
                           const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
                           long v_base, float scale, int split, int seg_chunks, float* part) {
     extern __shared__ float sm[];
@@ -688,6 +709,8 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
     const float* q = qs + qh * dimp;
     const int pw = dim + vdim;
     const bool kvec = (dim % (sizeof(T) == 2 ? 8 : 4)) == 0, pvec = (dim % 4 == 0) && (pw % 4 == 0);
+    const bool pair = sizeof(T) == 2 && (vdim % 2 == 0) && (dim % 2 == 0);
+    const bool coop = (dim % 8 == 0) && (pw % 4 == 0);
     float m = -INFINITY, l = 0.f, acc[HB_MAX_VPL];
 #pragma unroll
     for (int e = 0; e < HB_MAX_VPL; ++e) acc[e] = 0.f;
@@ -695,37 +718,137 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
     float* wpr = pr + wv * 64;
     for (int base = (c0 + sp) * 64; base < c1 * 64; base += split * 64) {
         const int u = base + lane;
-        float sc = -INFINITY;
+        const int cnt = total - base < 64 ? total - base : 64;
+        // where each lane's own key lives: >= 0 a token of the cache, < 0 a pooled entry
         long where = 0;
         if (u < total) {
-            float dot;
             if (u < nb) {
                 const int t = u * P + P - 1;
-                const size_t entry = ((size_t)pt[t / ps] * ppp + (t % ps) / P) * G + g;
-                dot = hb_dot_row(q, pool + entry * pw, dim, pvec);
-                where = -(long)entry - 1;
+                where = -(long)(((size_t)pt[t / ps] * ppp + (t % ps) / P) * G + g) - 1;
             } else {
                 const int j = lo + (u - nb);
-                const size_t tok = (size_t)pt[j / ps] * ps + j % ps;
-                dot = hb_dot_row(q, cache + tok * (size_t)(G * dim) + g * dim, dim, kvec);
-                where = (long)tok;
+                where = (long)((size_t)pt[j / ps] * ps + j % ps);
             }
-            sc = dot * scale;
         }
+        __builtin_amdgcn_wave_barrier();
+        wloc[lane] = where;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        float dot = 0.f;
+        const int npool_c = nb - base < 0 ? 0 : (nb - base < cnt ? nb - base : cnt);
+        if (coop && sizeof(T) == 2 && dim <= 128 && npool_c == 0) {
+            // a chunk of cached tokens only, one 128-dim slice: all sixteen row requests of the wave go out before the first is used
+            const int sub = lane & 15, grp = lane >> 4;
+            const bool mine_ok = sub * 8 < dim;
+            const bf16_t* kb = (const bf16_t*)cache + g * dim + (mine_ok ? sub * 8 : 0);
+            float4 qa = make_float4(0.f, 0.f, 0.f, 0.f), qb = qa;
+            if (mine_ok) { qa = *(const float4*)(q + sub * 8); qb = *(const float4*)(q + sub * 8 + 4); }
+#pragma unroll
+            for (int half = 0; half < 2; ++half) {
+                uint4 kreg[8];
+#pragma unroll
+                for (int i8 = 0; i8 < 8; ++i8) {
+                    const int it = half * 8 + i8;
+                    const int kk = it * 4 + grp < cnt ? it * 4 + grp : cnt - 1;
+                    kreg[i8] = *(const uint4*)(kb + (size_t)wloc[kk] * (size_t)(G * dim));
+                }
+#pragma unroll
+                for (int i8 = 0; i8 < 8; ++i8) {
+                    const int it = half * 8 + i8;
+                    const uint4 u4 = kreg[i8];
+                    float part = 0.f;
+                    part = fmaf(qa.x, bflo(u4.x), part); part = fmaf(qa.y, bfhi(u4.x), part); part = fmaf(qa.z, bflo(u4.y), part); part = fmaf(qa.w, bfhi(u4.y), part);
+                    part = fmaf(qb.x, bflo(u4.z), part); part = fmaf(qb.y, bfhi(u4.z), part); part = fmaf(qb.z, bflo(u4.w), part); part = fmaf(qb.w, bfhi(u4.w), part);
+                    part += __shfl_xor(part, 8, 64);
+                    part += __shfl_xor(part, 4, 64);
+                    part += __shfl_xor(part, 2, 64);
+                    part += __shfl_xor(part, 1, 64);
+                    const float got = __shfl(part, (lane & 3) * 16, 64);
+                    if ((lane >> 2) == it) dot = got;
+                }
+            }
+        } else if (coop) {
+            // sixteen lanes per key: each takes 8 dims of every 128 (one 16-byte request of a bf16 row), so a wave's request covers
+            // four whole key rows instead of 64 scattered ones; the 16 partial dots are added by a butterfly, then lane L takes key L's
+            const int sub = lane & 15, grp = lane >> 4;
+            for (int it = 0; it * 4 < cnt; ++it) {
+                const int kk = it * 4 + grp < cnt ? it * 4 + grp : cnt - 1;
+                const long w = wloc[kk];
+                float part = 0.f;
+                if (w < 0) {
+                    const float* kp = pool + (size_t)(-w - 1) * pw;
+                    for (int d = sub * 8; d < dim; d += 128) {
+                        const float4 k0 = *(const float4*)(kp + d), k1 = *(const float4*)(kp + d + 4);
+                        const float4 a = *(const float4*)(q + d), b2 = *(const float4*)(q + d + 4);
+                        part = fmaf(a.x, k0.x, part); part = fmaf(a.y, k0.y, part); part = fmaf(a.z, k0.z, part); part = fmaf(a.w, k0.w, part);
+                        part = fmaf(b2.x, k1.x, part); part = fmaf(b2.y, k1.y, part); part = fmaf(b2.z, k1.z, part); part = fmaf(b2.w, k1.w, part);
+                    }
+                } else {
+                    part = hb_dot_slices(q, cache + (size_t)w * (size_t)(G * dim) + g * dim, dim, sub);
+                }
+                part += __shfl_xor(part, 8, 64);
+                part += __shfl_xor(part, 4, 64);
+                part += __shfl_xor(part, 2, 64);
+                part += __shfl_xor(part, 1, 64);
+                const float got = __shfl(part, (lane & 3) * 16, 64);
+                if ((lane >> 2) == it) dot = got;
+            }
+        } else if (u < total) {
+            dot = where < 0 ? hb_dot_row(q, pool + (size_t)(-where - 1) * pw, dim, pvec)
+                            : hb_dot_row(q, cache + (size_t)where * (size_t)(G * dim) + g * dim, dim, kvec);
+        }
+        const float sc = u < total ? dot * scale : -INFINITY;
         const float mn = fmaxf(m, hb_wave_max(sc));
         const float alpha = expf(m - mn);
         const float e = u < total ? expf(sc - mn) : 0.f;
         l = l * alpha + hb_wave_sum(e);
         m = mn;
-        __builtin_amdgcn_wave_barrier();
         wpr[lane] = e;
-        wloc[lane] = where;
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        const int cnt = total - base < 64 ? total - base : 64;
-        // pooled keys come first in the key order: two loops without a per-key branch, eight independent requests in flight each
+        // pooled keys come first in the key order: two loops without a per-key branch, many independent requests in flight each.
+        // acc[e] belongs to value column hb_vcol(e): with a bf16 cache and an even vdim a lane owns two adjacent columns of each
+        // 128-column group (one 4-byte request per key), else one column of each 64-column group.
         const int npool = nb - base < 0 ? 0 : (nb - base < cnt ? nb - base : cnt);
         const size_t gv = (size_t)G * vdim;
+        if (pair) {
+#pragma unroll
+            for (int c = 0; c < HB_MAX_VPL / 2; ++c) {
+                if (c * 128 < vdim) {
+                    const int j = c * 128 + 2 * lane;
+                    const int jj = j < vdim ? j : vdim - 2;
+                    const float* pbase = pool + dim + jj;
+                    const T* vbase = cache + v_base + g * vdim + jj;
+                    float a0 = acc[2 * c] * alpha, a1 = acc[2 * c + 1] * alpha;
+                    for (int k0 = 0; k0 < npool; k0 += 8) {
+                        float pv[8];
+                        float2 vv[8];
+#pragma unroll
+                        for (int x = 0; x < 8; ++x) {
+                            const int kk = k0 + x < npool ? k0 + x : npool - 1;
+                            pv[x] = k0 + x < npool ? wpr[kk] : 0.f;
+                            vv[x] = *(const float2*)(pbase + (size_t)(-wloc[kk] - 1) * pw);
+                        }
+#pragma unroll
+                        for (int x = 0; x < 8; ++x) { a0 = fmaf(pv[x], vv[x].x, a0); a1 = fmaf(pv[x], vv[x].y, a1); }
+                    }
+                    for (int k0 = npool; k0 < cnt; k0 += 16) {
+                        float pv[16];
+                        u32 vv[16];
+#pragma unroll
+                        for (int x = 0; x < 16; ++x) {
+                            const int kk = k0 + x < cnt ? k0 + x : cnt - 1;
+                            pv[x] = k0 + x < cnt ? wpr[kk] : 0.f;
+                            vv[x] = *(const u32*)(vbase + (size_t)wloc[kk] * gv);
+                        }
+#pragma unroll
+                        for (int x = 0; x < 16; ++x) { a0 = fmaf(pv[x], bflo(vv[x]), a0); a1 = fmaf(pv[x], bfhi(vv[x]), a1); }
+                    }
+                    acc[2 * c] = a0;
+                    acc[2 * c + 1] = a1;
+                }
+            }
+        } else {
 #pragma unroll
         for (int c = 0; c < HB_MAX_VPL; ++c) {
             const int j = lane + c * 64;
@@ -745,27 +868,30 @@ __global__ void k_hb_attn(const float* proj, long ldp, const T* cache, const flo
 #pragma unroll
                     for (int x = 0; x < 8; ++x) a = fmaf(pv[x], vv[x], a);
                 }
-                for (int k0 = npool; k0 < cnt; k0 += 32) {
-                    float pv[32], vv[32];
+                for (int k0 = npool; k0 < cnt; k0 += 16) {
+                    float pv[16], vv[16];
 #pragma unroll
-                    for (int x = 0; x < 32; ++x) {
+                    for (int x = 0; x < 16; ++x) {
                         const int kk = k0 + x < cnt ? k0 + x : cnt - 1;
                         pv[x] = k0 + x < cnt ? wpr[kk] : 0.f;
                         vv[x] = hb_ld(vbase + (size_t)wloc[kk] * gv);
                     }
 #pragma unroll
-                    for (int x = 0; x < 32; ++x) a = fmaf(pv[x], vv[x], a);
+                    for (int x = 0; x < 16; ++x) a = fmaf(pv[x], vv[x], a);
                 }
                 acc[c] = a;
             }
+        }
         }
         __builtin_amdgcn_wave_barrier();
     }
     // merge the splits of each head in split order
     float* mine = mo + (size_t)wv * (vdim + 2);
 #pragma unroll
-    for (int c = 0; c < HB_MAX_VPL; ++c)
-        if (lane + c * 64 < vdim) mine[lane + c * 64] = acc[c];
+    for (int c = 0; c < HB_MAX_VPL; ++c) {
+        const int j = pair ? (c >> 1) * 128 + 2 * lane + (c & 1) : lane + c * 64;
+        if (j < vdim) mine[j] = acc[c];
+    }
     if (lane == 0) { mine[vdim] = m; mine[vdim + 1] = l; }
     __syncthreads();
     if (sp == 0) {
@@ -927,7 +1053,7 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
                                io->page, io->slot, H, G, L.dim, L.vdim, L.rot_dims, ps, v_base, c.eps);
             hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)run.cache, run.pool, io->pos, io->row_req,
                                io->page_table, io->pt_stride, G, L.dim, L.vdim, L.pool, ps, ppp, v_base);
-            const int split = QG >= 8 ? 1 : (QG >= 4 ? 2 : 4);
+            const int split = 16 / QG >= 4 ? 4 : (16 / QG >= 1 ? 16 / QG : 1);      // up to 16 waves per block, at most 4 per head
             const int nwv2 = QG * split, dimp = (L.dim + 3) & ~3;
             const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (L.vdim + 2) * 4;
             // steps of few rows: 4-chunk key segments on separate blocks + a merge pass (more blocks than rows x kv heads); a row's

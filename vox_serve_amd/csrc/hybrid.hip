@@ -416,15 +416,22 @@ int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const
 // (dim, DPW) only, never on how the tokens are cut into steps.
 #define HB_SCAN_MAX_WAVES 16
 
+// The inputs of TT tokens at a time are staged in LDS by the whole block (activations applied there, one memory round trip per
+// tile instead of one per token); TT only groups requests, it does not enter any sum.
 // HGRN2: S_t = diag(f_t) S_{t-1} + (1 - f_t) v_t^T,  o_t = S_t^T q_t.
 // proj row = [q (H*dim) | f (H*dim) | v (H*vdim)] pre-activation (bias already added).
 template <int DPW>
 __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_hgrn2_scan(const float* proj, long ldp, float* out, long ldo, const float* lower,
                                                                           float* state, const int* req_rows, const int* req_state,
-                                                                          const int* pos, int H, int dim, int vdim) {
-    __shared__ float fs[HB_SCAN_MAX_WAVES * DPW], qs[HB_SCAN_MAX_WAVES * DPW], part[HB_SCAN_MAX_WAVES][64];
+                                                                          const int* pos, int H, int dim, int vdim, int TT) {
+    extern __shared__ float sm[];
+    const int nw = blockDim.x >> 6, dpad = nw * DPW;
+    float* fs = sm;                       // [TT][dpad]
+    float* qs = fs + TT * dpad;           // [TT][dpad]
+    float* vs = qs + TT * dpad;           // [TT][64]
+    float* part = vs + TT * 64;           // [2][nw][64]
     const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.z * 64 + lane;
-    const int nw = blockDim.x >> 6, d0 = w * DPW;
+    const int d0 = w * DPW;
     const int rs = req_rows[r], re = req_rows[r + 1];
     if (rs >= re) return;
     const bool ok = c < vdim, fresh = pos[rs] == 0;
@@ -432,34 +439,48 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_hgrn2_scan(const 
     float S[DPW];
 #pragma unroll
     for (int i = 0; i < DPW; ++i) S[i] = (ok && !fresh && d0 + i < dim) ? St[(size_t)(d0 + i) * vdim + c] : 0.f;
-    for (int t = rs; t < re; ++t) {
-        const float* p = proj + (size_t)t * ldp;
-        for (int d = threadIdx.x; d < nw * DPW; d += blockDim.x) {
+    int flip = 0;
+    for (int t0 = rs; t0 < re; t0 += TT) {
+        const int nt = re - t0 < TT ? re - t0 : TT;
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nt * dpad; idx += blockDim.x) {
+            const int tt = idx / dpad, d = idx - tt * dpad;
             float q = 0.f, f = 0.f;
             if (d < dim) {
+                const float* p = proj + (size_t)(t0 + tt) * ldp;
                 const float qv = p[h * dim + d], lo = lower[h * dim + d];
                 q = qv * hb_sigmoid(qv);
                 f = lo + (1.0f - lo) * hb_sigmoid(p[H * dim + h * dim + d]);
             }
-            qs[d] = q;
-            fs[d] = f;
+            qs[idx] = q;
+            fs[idx] = f;
         }
-        const float v = ok ? p[2 * H * dim + h * vdim + c] : 0.f;
+        for (int idx = threadIdx.x; idx < nt * 64; idx += blockDim.x) {
+            const int tt = idx >> 6, cc = blockIdx.z * 64 + (idx & 63);
+            vs[idx] = cc < vdim ? proj[(size_t)(t0 + tt) * ldp + 2 * H * dim + h * vdim + cc] : 0.f;
+        }
         __syncthreads();
-        float o = 0.f;
+        for (int tt = 0; tt < nt; ++tt) {
+            const float v = vs[tt * 64 + lane];
+            const float* ft = fs + tt * dpad + d0;
+            const float* qt = qs + tt * dpad + d0;
+            float o = 0.f;
 #pragma unroll
-        for (int i = 0; i < DPW; ++i) {
-            const float f = fs[d0 + i];
-            const float sv = f * S[i] + (1.0f - f) * v;
-            S[i] = sv;
-            o = fmaf(sv, qs[d0 + i], o);
-        }
-        part[w][lane] = o;
-        __syncthreads();
-        if (w == 0 && ok) {
-            float sum = part[0][lane];
-            for (int k = 1; k < nw; ++k) sum += part[k][lane];
-            out[(size_t)t * ldo + h * vdim + c] = sum;
+            for (int i = 0; i < DPW; ++i) {
+                const float f = ft[i];
+                const float sv = f * S[i] + (1.0f - f) * v;
+                S[i] = sv;
+                o = fmaf(sv, qt[i], o);
+            }
+            float* pt = part + flip * nw * 64;
+            pt[w * 64 + lane] = o;
+            __syncthreads();
+            if (w == 0 && ok) {
+                float sum = pt[lane];
+                for (int k = 1; k < nw; ++k) sum += pt[k * 64 + lane];
+                out[(size_t)(t0 + tt) * ldo + h * vdim + c] = sum;
+            }
+            flip ^= 1;
         }
     }
     if (ok)
@@ -474,65 +495,88 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_hgrn2_scan(const 
 template <int DPW>
 __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_mlstm_scan(const float* proj, long ldp, float* out, long ldo, float* state,
                                                                           const int* req_rows, const int* req_state, const int* pos, int H,
-                                                                          int dim, int vdim, float cap) {
-    __shared__ float ks[HB_SCAN_MAX_WAVES * DPW], qs[HB_SCAN_MAX_WAVES * DPW], part[HB_SCAN_MAX_WAVES][64], npart[HB_SCAN_MAX_WAVES];
+                                                                          int dim, int vdim, float cap, int TT) {
+    extern __shared__ float sm[];
+    const int nw = blockDim.x >> 6, dpad = nw * DPW;
+    float* ks = sm;                       // [TT][dpad]
+    float* qs = ks + TT * dpad;           // [TT][dpad]
+    float* vs = qs + TT * dpad;           // [TT][64]
+    float* gs = vs + TT * 64;             // [TT][2]: log input gate, log forget gate
+    float* part = gs + TT * 2;            // [2][nw][65]: partial outputs and (column 64) partial n.q
     const int r = blockIdx.x, h = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.z * 64 + lane;
-    const int nw = blockDim.x >> 6, d0 = w * DPW;
+    const int d0 = w * DPW;
     const int rs = req_rows[r], re = req_rows[r + 1];
     if (rs >= re) return;
     const bool ok = c < vdim, fresh = pos[rs] == 0;
     const size_t per = (size_t)dim * vdim + dim + 1;
     float* St = state + ((size_t)req_state[r] * H + h) * per;
-    float* nt = St + (size_t)dim * vdim;
+    float* nt_ = St + (size_t)dim * vdim;
     float S[DPW], nn[DPW];
 #pragma unroll
     for (int i = 0; i < DPW; ++i) {
         S[i] = (ok && !fresh && d0 + i < dim) ? St[(size_t)(d0 + i) * vdim + c] : 0.f;
-        nn[i] = (!fresh && d0 + i < dim) ? nt[d0 + i] : 0.f;
+        nn[i] = (!fresh && d0 + i < dim) ? nt_[d0 + i] : 0.f;
     }
-    float m = fresh ? 0.f : nt[dim];
+    float m = fresh ? 0.f : nt_[dim];
     const float qscale = 1.0f / sqrtf((float)dim);
     const int off_k = H * dim, off_v = 2 * H * dim, off_i = 2 * H * dim + 2 * H * vdim, off_f = off_i + H;
-    for (int t = rs; t < re; ++t) {
-        const float* p = proj + (size_t)t * ldp;
-        for (int d = threadIdx.x; d < nw * DPW; d += blockDim.x) {
-            ks[d] = d < dim ? p[off_k + h * dim + d] : 0.f;
-            qs[d] = d < dim ? p[h * dim + d] * qscale : 0.f;
-        }
-        const float ig = cap * tanhf(p[off_i + h] / cap);
-        const float fg = hb_logsigmoid(cap * tanhf(p[off_f + h] / cap));
-        const float mn = fmaxf(fg + m, ig);
-        const float a = expf(fg + m - mn), b = expf(ig - mn);
-        const float v = ok ? p[off_v + h * vdim + c] : 0.f;
-        const float bv = b * v;
+    int flip = 0;
+    for (int t0 = rs; t0 < re; t0 += TT) {
+        const int nt = re - t0 < TT ? re - t0 : TT;
         __syncthreads();
-        float o = 0.f, nq = 0.f;
+        for (int idx = threadIdx.x; idx < nt * dpad; idx += blockDim.x) {
+            const int tt = idx / dpad, d = idx - tt * dpad;
+            const float* p = proj + (size_t)(t0 + tt) * ldp;
+            ks[idx] = d < dim ? p[off_k + h * dim + d] : 0.f;
+            qs[idx] = d < dim ? p[h * dim + d] * qscale : 0.f;
+        }
+        for (int idx = threadIdx.x; idx < nt * 64; idx += blockDim.x) {
+            const int tt = idx >> 6, cc = blockIdx.z * 64 + (idx & 63);
+            vs[idx] = cc < vdim ? proj[(size_t)(t0 + tt) * ldp + off_v + h * vdim + cc] : 0.f;
+        }
+        for (int tt = threadIdx.x; tt < nt; tt += blockDim.x) {
+            const float* p = proj + (size_t)(t0 + tt) * ldp;
+            gs[2 * tt] = cap * tanhf(p[off_i + h] / cap);
+            gs[2 * tt + 1] = hb_logsigmoid(cap * tanhf(p[off_f + h] / cap));
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float ig = gs[2 * tt], fg = gs[2 * tt + 1];
+            const float mn = fmaxf(fg + m, ig);
+            const float a = expf(fg + m - mn), b = expf(ig - mn);
+            const float bv = b * vs[tt * 64 + lane];
+            const float* kt = ks + tt * dpad + d0;
+            const float* qt = qs + tt * dpad + d0;
+            float o = 0.f, nq = 0.f;
 #pragma unroll
-        for (int i = 0; i < DPW; ++i) {
-            const float kv = ks[d0 + i], qv = qs[d0 + i];
-            nn[i] = a * nn[i] + b * kv;
-            nq = fmaf(nn[i], qv, nq);
-            const float sv = a * S[i] + kv * bv;
-            S[i] = sv;
-            o = fmaf(sv, qv, o);
-        }
-        part[w][lane] = o;
-        if (lane == 0) npart[w] = nq;
-        m = mn;
-        __syncthreads();
-        if (w == 0 && ok) {
-            float sum = part[0][lane], nsum = npart[0];
-            for (int k = 1; k < nw; ++k) { sum += part[k][lane]; nsum += npart[k]; }
-            out[(size_t)t * ldo + h * vdim + c] = sum / (fmaxf(fabsf(nsum), expf(-m)) + 1e-6f);
+            for (int i = 0; i < DPW; ++i) {
+                const float kv = kt[i], qv = qt[i];
+                nn[i] = a * nn[i] + b * kv;
+                nq = fmaf(nn[i], qv, nq);
+                const float sv = a * S[i] + kv * bv;
+                S[i] = sv;
+                o = fmaf(sv, qv, o);
+            }
+            float* pt = part + flip * nw * 65;
+            pt[w * 65 + lane] = o;
+            if (lane == 0) pt[w * 65 + 64] = nq;
+            m = mn;
+            __syncthreads();
+            if (w == 0 && ok) {
+                float sum = pt[lane], nsum = pt[64];
+                for (int k = 1; k < nw; ++k) { sum += pt[k * 65 + lane]; nsum += pt[k * 65 + 64]; }
+                out[(size_t)(t0 + tt) * ldo + h * vdim + c] = sum / (fmaxf(fabsf(nsum), expf(-m)) + 1e-6f);
+            }
+            flip ^= 1;
         }
     }
 #pragma unroll
     for (int i = 0; i < DPW; ++i)
         if (d0 + i < dim) {
             if (ok) St[(size_t)(d0 + i) * vdim + c] = S[i];
-            if (blockIdx.z == 0 && lane == 0) nt[d0 + i] = nn[i];
+            if (blockIdx.z == 0 && lane == 0) nt_[d0 + i] = nn[i];
         }
-    if (blockIdx.z == 0 && threadIdx.x == 0) nt[dim] = m;
+    if (blockIdx.z == 0 && threadIdx.x == 0) nt_[dim] = m;
 }
 
 // per (row, head): o / rms(o) over vdim, times a weight (per_head_w: indexed over all heads, else shared [vdim]), times
@@ -1033,16 +1077,21 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
         // dims per wave of the scans: the smallest of 16 / 32 / 64 that covers dim with at most 16 waves
         const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
         const int nwv = (L.dim + dpw - 1) / dpw;
+        // tokens staged per tile: as many as fit 4096 staged floats per array, at most 16
+        const int dpad = nwv * dpw;
+        const int tt = 4096 / dpad >= 16 ? 16 : (4096 / dpad >= 1 ? 4096 / dpad : 1);
         if (L.kind == VOX_MIXER_HGRN2) {
             auto kern = dpw == 16 ? k_hb_hgrn2_scan<16> : (dpw == 32 ? k_hb_hgrn2_scan<32> : k_hb_hgrn2_scan<64>);
-            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), 0, st, m->proj, (long)n_in, m->mix, (long)n_mix, L.lower,
-                               run.state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim);
+            const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + 2 * nwv * 64) * 4;
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, L.lower,
+                               run.state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, tt);
             hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 0, m->proj, (long)n_in, -1,
                                L.vdim, c.eps);
         } else if (L.kind == VOX_MIXER_MLSTM) {
             auto kern = dpw == 16 ? k_hb_mlstm_scan<16> : (dpw == 32 ? k_hb_mlstm_scan<32> : k_hb_mlstm_scan<64>);
-            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), 0, st, m->proj, (long)n_in, m->mix, (long)n_mix, run.state,
-                               io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap);
+            const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + tt * 2 + 2 * nwv * 65) * 4;
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, run.state,
+                               io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap, tt);
             hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_in,
                                2 * L.heads * L.dim + L.heads * L.vdim, L.vdim, c.eps);
         } else {

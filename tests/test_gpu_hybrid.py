@@ -242,6 +242,20 @@ def test_wide_sizes():
     check(cfg, S, toks, [80], dtype=torch.bfloat16)
 
 
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_odd_sizes(dtype):
+    """Sizes that defeat every vector path: width 18, key dims 10 / 5 / 3, value dims 6 / 7 / 5, 3 query heads per K/V head,
+    6 of 10 dims rotated, a 37-entry vocabulary, a window of 11 and blocks of 5 on pages of 8."""
+    layers = [U.hgrn2(heads=3, dim=5, vdim=7, ff=13), U.attention(heads=3, kv_heads=1, dim=10, vdim=6, window=11, pool=5, rot=6, ff=0),
+              U.mlstm(heads=1, dim=3, vdim=5), U.attention(heads=2, kv_heads=2, dim=6, vdim=9, window=2, pool=7, rot=2, factor=3.0)]
+    cfg = U.config(layers, width=18, vocab=37, loop=(1, 4, 2))
+    S = U.random_checkpoint(cfg, seed=51)
+    toks = tokens(75, 37, 52)
+    q = None if dtype == torch.float32 else 0.9
+    check(cfg, S, toks, [75], dtype=dtype, quantile=q)
+    check(cfg, S, toks, [9, 2, 33, 5], dtype=dtype, quantile=q)
+
+
 def test_greedy_generation_through_the_scheduler():
     """Requests enter through the scheduler's transport, are prefilled in portions next to decoding requests and generate greedily;
     the ids equal the oracle's greedy continuation (fp32 engine)."""

@@ -242,6 +242,15 @@ def test_wide_sizes():
     check(cfg, S, toks, [80], dtype=torch.bfloat16)
 
 
+def test_large_recurrent_dims():
+    """Key dims beyond 256 per head: the scans keep 32 dims per wave instead of 16, and stage fewer tokens per tile."""
+    cfg = U.config([U.hgrn2(heads=1, dim=300, vdim=24), U.mlstm(heads=2, dim=272, vdim=16)], width=32, vocab=40)
+    S = U.random_checkpoint(cfg, seed=55)
+    toks = tokens(50, 40, 56)
+    check(cfg, S, toks, [50])
+    check(cfg, S, toks, [17, 2, 20])
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_odd_sizes(dtype):
     """Sizes that defeat every vector path: width 18, key dims 10 / 5 / 3, value dims 6 / 7 / 5, 3 query heads per K/V head,

@@ -64,30 +64,64 @@ __global__ __launch_bounds__(256) void k_hb_embed(const T* table, const int* ids
 }
 
 // ---- layer norm with a weight and no bias, fp32; optional row gather ----------------------------------------------------
+// mean, then the mean of the squared deviations (two passes over the row).  NV > 0: the row (width <= 256 * NV) is read once
+// into registers; NV = 0: any width, three reads.  Same sums in the same order either way.
+template <int NV>
 __global__ __launch_bounds__(256) void k_hb_layernorm(const float* x, long ldx, const int* rows, const float* w, float* y, long ldy, int W,
                                                       float eps) {
-    __shared__ float red[4];
+    __shared__ float red[2][4];
     const int r = blockIdx.x, src = rows ? rows[r] : r;
     const float* xr = x + (size_t)src * ldx;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    float xv[NV > 0 ? NV : 1];
     float s = 0.f;
-    for (int i = threadIdx.x; i < W; i += 256) s += xr[i];
+    if (NV > 0) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int k = threadIdx.x + i * 256;
+            xv[i] = k < W ? xr[k] : 0.f;
+        }
+#pragma unroll
+        for (int i = 0; i < NV; ++i) s += xv[i];
+    } else {
+        for (int i = threadIdx.x; i < W; i += 256) s += xr[i];
+    }
     s = hb_wave_sum(s);
-    if (lane == 0) red[wv] = s;
+    if (lane == 0) red[0][wv] = s;
     __syncthreads();
-    const float mean = (((red[0] + red[1]) + red[2]) + red[3]) / (float)W;
-    __syncthreads();
+    const float mean = (((red[0][0] + red[0][1]) + red[0][2]) + red[0][3]) / (float)W;
     float q = 0.f;
-    for (int i = threadIdx.x; i < W; i += 256) {
-        const float d = xr[i] - mean;
-        q += d * d;
+    if (NV > 0) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const float d = threadIdx.x + i * 256 < W ? xv[i] - mean : 0.f;
+            q += d * d;
+        }
+    } else {
+        for (int i = threadIdx.x; i < W; i += 256) {
+            const float d = xr[i] - mean;
+            q += d * d;
+        }
     }
     q = hb_wave_sum(q);
-    if (lane == 0) red[wv] = q;
+    if (lane == 0) red[1][wv] = q;
     __syncthreads();
-    const float var = (((red[0] + red[1]) + red[2]) + red[3]) / (float)W;
+    const float var = (((red[1][0] + red[1][1]) + red[1][2]) + red[1][3]) / (float)W;
     const float inv = 1.0f / sqrtf(var + eps);
-    for (int i = threadIdx.x; i < W; i += 256) y[(size_t)r * ldy + i] = (xr[i] - mean) * inv * w[i];
+    if (NV > 0) {
+#pragma unroll
+        for (int i = 0; i < NV; ++i) {
+            const int k = threadIdx.x + i * 256;
+            if (k < W) y[(size_t)r * ldy + k] = (xv[i] - mean) * inv * w[k];
+        }
+    } else {
+        for (int i = threadIdx.x; i < W; i += 256) y[(size_t)r * ldy + i] = (xr[i] - mean) * inv * w[i];
+    }
+}
+static void hb_layernorm(hipStream_t st, int n, const float* x, long ldx, const int* rows, const float* w, float* y, long ldy, int W, float eps) {
+    if (W <= 1024) hipLaunchKernelGGL(k_hb_layernorm<4>, dim3(n), dim3(256), 0, st, x, ldx, rows, w, y, ldy, W, eps);
+    else if (W <= 4096) hipLaunchKernelGGL(k_hb_layernorm<16>, dim3(n), dim3(256), 0, st, x, ldx, rows, w, y, ldy, W, eps);
+    else hipLaunchKernelGGL(k_hb_layernorm<0>, dim3(n), dim3(256), 0, st, x, ldx, rows, w, y, ldy, W, eps);
 }
 
 // ---- GEMM  C[M,N] (+)= A[M,K] . W[N,K]^T + bias ---------------------------------------------------------------------------
@@ -1071,7 +1105,7 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             float* t = cur; cur = other; other = t;
         }
         const int n_in = hb_layer_in(L), n_mix = L.heads * L.vdim;
-        hipLaunchKernelGGL(k_hb_layernorm, dim3(n), dim3(256), 0, st, cur, ldx, (const int*)nullptr, L.norm1, m->h, (long)W, W, c.eps);
+        hb_layernorm(st, n, cur, ldx, nullptr, L.norm1, m->h, (long)W, W, c.eps);
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->h, W, (const T*)L.w_in, L.b_in, m->proj, n_in, n, n_in, W));
         const int vt = (L.vdim + 63) / 64;
         // dims per wave of the scans: the smallest of 16 / 32 / 64 that covers dim with at most 16 waves
@@ -1119,7 +1153,7 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
         }
         VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix));
         if (L.ff > 0) {
-            hipLaunchKernelGGL(k_hb_layernorm, dim3(n), dim3(256), 0, st, cur, ldx, (const int*)nullptr, L.norm2, m->h, (long)W, W, c.eps);
+            hb_layernorm(st, n, cur, ldx, nullptr, L.norm2, m->h, (long)W, W, c.eps);
             VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
             VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff, L.ff, (const T*)L.w_down, nullptr, cur, ldx, n, W, L.ff));
         }
@@ -1127,7 +1161,7 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
     }
     if (n_out > 0) {
-        hipLaunchKernelGGL(k_hb_layernorm, dim3(n_out), dim3(256), 0, st, cur, ldx, io->out_rows, m->w.final_norm, m->hout, (long)W, W, c.eps);
+        hb_layernorm(st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, (long)W, W, c.eps);
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits, c.vocab, n_out, c.vocab, W));
     }
     VOX_HIP(hipGetLastError());

@@ -305,3 +305,44 @@ def test_greedy_generation_through_the_scheduler():
         assert worker.empty_pages.qsize() == 64 and worker.empty_state_slots.qsize() == 4
     finally:
         model.engine.close()
+
+
+def test_top_k_sampling_through_the_scheduler():
+    """Stochastic sampling goes through the library's sampler: every generated id is one of the oracle's five most likely
+    continuations of the request's own prefix, and a second run with the same seed repeats the ids."""
+    from vox_serve_amd.model.sirodra import SirodraModel, config_from_dict
+    from vox_serve_amd.sampling import SamplingConfig
+    from vox_serve_amd.scheduler.base import Scheduler, encode_request
+    from vox_serve_amd.worker.base import ModelWorker
+    cfg = stack(sharp=False)
+    S = U.random_checkpoint(cfg, seed=61)
+    prompts = {"a": tokens(21, 64, 62), "b": tokens(9, 64, 63)}
+
+    def generate():
+        model = SirodraModel("sirodra-test", S, config_from_dict(cfg), dtype=torch.float32, max_batch_size=2, page_size=8, max_num_pages=32,
+                             max_seq_len=256, max_prefill_tokens=64, state_slots=2, max_tokens=10,
+                             sampling=SamplingConfig(top_k=5, temperature=0.8, max_tokens=10))
+        worker = ModelWorker(model=model, max_batch_size=2, max_num_pages=32, page_size=8, seed=7)
+        sched = Scheduler(worker, max_batch_size=2)
+        try:
+            for rid, p in prompts.items():
+                sched.transport.requests.put(encode_request(rid, " ".join(map(str, p)), is_streaming=False))
+            reqs = {}
+            for _ in range(200):
+                sched._step()
+                for r in sched.active_requests:
+                    reqs[r.request_id] = r
+                if not sched.active_requests and not sched.transport.pending():
+                    break
+            return {rid: [int(t[0, 0]) for t in reqs[rid].lm_output_tokens] for rid in prompts}
+        finally:
+            model.engine.close()
+    first = generate()
+    for rid, p in prompts.items():
+        assert len(first[rid]) == 10
+        seq = list(p)
+        for tok in first[rid]:
+            top = HR.forward(cfg, S, seq)[-1].topk(5).indices.tolist()
+            assert tok in top, (rid, tok, top)
+            seq.append(tok)
+    assert generate() == first

@@ -342,6 +342,91 @@ __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const
         }
 }
 
+// One-row steps: the weight-only LayerNorm of the row fused in front of the GEMV.  Every wave takes the row's statistics itself
+// (mean, then the mean of the squared deviations; lane-chunked sums and a butterfly, an order fixed by K), so the row is read three
+// times from cache instead of once from a normalised copy, and a dependent launch is saved.  Needs K % 8 == 0 (4 for fp32).
+template <typename T, int EPI, int CPW>
+__global__ __launch_bounds__(256) void k_hb_ln_gemv(const float* X, long ldx, const int* rows, const float* lnw, float eps, const T* Wt,
+                                                    const float* bias, float* C, int N, int K) {
+    const int lane = threadIdx.x & 63, n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * CPW;
+    if (n0 >= N) return;
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    const float* xr = X + (size_t)(rows ? rows[0] : 0) * ldx;
+    float s = 0.f;
+    for (int k = lane * CH; k < K; k += 64 * CH)
+#pragma unroll
+        for (int e = 0; e < CH; e += 4) {
+            const float4 x4 = *(const float4*)(xr + k + e);
+            s += x4.x; s += x4.y; s += x4.z; s += x4.w;
+        }
+    const float mean = hb_wave_sum(s) / (float)K;
+    float q = 0.f;
+    for (int k = lane * CH; k < K; k += 64 * CH)
+#pragma unroll
+        for (int e = 0; e < CH; e += 4) {
+            const float4 x4 = *(const float4*)(xr + k + e);
+            const float d0 = x4.x - mean, d1 = x4.y - mean, d2 = x4.z - mean, d3 = x4.w - mean;
+            q += d0 * d0; q += d1 * d1; q += d2 * d2; q += d3 * d3;
+        }
+    const float inv = 1.0f / sqrtf(hb_wave_sum(q) / (float)K + eps);
+    float acc[CPW];
+#pragma unroll
+    for (int j = 0; j < CPW; ++j) acc[j] = 0.f;
+    const T* wr[CPW];
+#pragma unroll
+    for (int j = 0; j < CPW; ++j) wr[j] = Wt + (size_t)(n0 + j < N ? n0 + j : N - 1) * K;
+    for (int k = lane * CH; k < K; k += 64 * CH) {
+        float w[CPW][CH];
+#pragma unroll
+        for (int j = 0; j < CPW; ++j) {
+            if (sizeof(T) == 2) {
+                const uint4 u = *(const uint4*)(wr[j] + k);
+                w[j][0] = bflo(u.x); w[j][1] = bfhi(u.x); w[j][2] = bflo(u.y); w[j][3] = bfhi(u.y);
+                if (CH == 8) { w[j][4] = bflo(u.z); w[j][5] = bfhi(u.z); w[j][6] = bflo(u.w); w[j][7] = bfhi(u.w); }
+            } else {
+                const float4 u = *(const float4*)(wr[j] + k);
+                w[j][0] = u.x; w[j][1] = u.y; w[j][2] = u.z; w[j][3] = u.w;
+            }
+        }
+#pragma unroll
+        for (int e = 0; e < CH; e += 4) {
+            const float4 x4 = *(const float4*)(xr + k + e), g4 = *(const float4*)(lnw + k + e);
+            const float x[4] = {hb_operand<T>((x4.x - mean) * inv * g4.x), hb_operand<T>((x4.y - mean) * inv * g4.y),
+                                hb_operand<T>((x4.z - mean) * inv * g4.z), hb_operand<T>((x4.w - mean) * inv * g4.w)};
+#pragma unroll
+            for (int j = 0; j < CPW; ++j) {
+                acc[j] = fmaf(w[j][e], x[0], acc[j]);
+                acc[j] = fmaf(w[j][e + 1], x[1], acc[j]);
+                acc[j] = fmaf(w[j][e + 2], x[2], acc[j]);
+                acc[j] = fmaf(w[j][e + 3], x[3], acc[j]);
+            }
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < CPW; ++j) {
+        const float sum = hb_wave_sum(acc[j]);
+        if (n0 + j < N && lane == 0) hb_epilogue<EPI>(C + n0 + j, sum, bias ? bias[n0 + j] : 0.f);
+    }
+}
+// true: the fused form was launched (one row, aligned operands); false: the caller normalises and multiplies in two launches
+template <typename T>
+bool hb_try_ln_gemv(hipStream_t st, int epi, const float* X, long ldx, const int* rows, const float* lnw, float eps, const T* W, const float* bias,
+                    float* C, int N, int K) {
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    if (K % CH || (ldx & 3) || ((size_t)X & 15) || ((size_t)W & 15) || ((size_t)lnw & 15)) return false;
+    const bool wide = N >= 16 * 1024;
+    const dim3 g(wide ? (N + 15) / 16 : (N + 3) / 4), b(256);
+#define HB_LN(EPI_) \
+    do { \
+        if (wide) hipLaunchKernelGGL((k_hb_ln_gemv<T, EPI_, 4>), g, b, 0, st, X, ldx, rows, lnw, eps, W, bias, C, N, K); \
+        else hipLaunchKernelGGL((k_hb_ln_gemv<T, EPI_, 1>), g, b, 0, st, X, ldx, rows, lnw, eps, W, bias, C, N, K); \
+    } while (0)
+    if (epi == HB_EPI_GELU) HB_LN(HB_EPI_GELU);
+    else HB_LN(HB_EPI_STORE);
+#undef HB_LN
+    return true;
+}
+
 // 2..16 rows, bf16: one MFMA row tile; a block owns 16 output columns and its four waves take the 32-wide k-steps w, w + 4, ...
 // with both fragments straight from memory (the weight fragment is one 16-byte request per lane, the activation fragment two,
 // converted to bf16 in registers); the four partial tiles are added in wave order.  Needs K % 32 == 0.
@@ -635,7 +720,8 @@ __global__ __launch_bounds__(64) void k_hb_head_norm(float* o, long ldo, const f
 #define HB_MAX_DPL 8   // dims per lane: dim <= 512
 template <typename T>
 __global__ __launch_bounds__(64) void k_hb_attn_prep(float* proj, long ldp, T* cache, const float* inv_freq, const int* pos, const int* page,
-                                                     const int* slot, int H, int G, int dim, int vdim, int rot, int ps, long v_base, float eps) {
+                                                     const int* slot, int H, int G, int dim, int vdim, int rot, int ps, long v_base, float eps,
+                                                     float* pool, const int* row_req, const int* ptab, int pts, int P, int ppp) {
     const int row = blockIdx.x, hb = blockIdx.y, lane = threadIdx.x;
     const bool is_q = hb < H;
     const int g = hb - H;
@@ -675,6 +761,31 @@ __global__ __launch_bounds__(64) void k_hb_attn_prep(float* proj, long ldp, T* c
     if (!is_q) {
         const float* vs = proj + (size_t)row * ldp + H * dim + G * dim + g * vdim;
         for (int j = lane; j < vdim; j += 64) hb_st(cache + v_base + tok * (size_t)(G * vdim) + g * vdim + j, vs[j]);
+        // steps with one row per request (pool != NULL): the pooled entry of a block this token closes, here instead of in a launch
+        // of its own — the block's other tokens were cached by earlier steps; this row's own values enter as the cache rounds them,
+        // last, which is k_hb_pool_update's arithmetic
+        const int pi = pos[row];
+        if (pool && (pi + 1) % P == 0) {
+            const int* pt = ptab + (size_t)row_req[row] * pts;
+            float* dst = pool + (((size_t)pt[pi / ps] * ppp + (pi % ps) / P) * G + g) * (size_t)(dim + vdim);
+#pragma unroll
+            for (int e = 0; e < HB_MAX_DPL; ++e) {
+                const int d = lane + e * 64;
+                if (d < dim) {
+                    float sum = 0.f;
+                    for (int j = pi - P + 1; j < pi; ++j) sum += hb_ld(cache + ((size_t)pt[j / ps] * ps + j % ps) * (size_t)(G * dim) + g * dim + d);
+                    sum += hb_operand<T>(y[e] * inv);
+                    dst[d] = sum / (float)P;
+                }
+            }
+            for (int j2 = lane; j2 < vdim; j2 += 64) {
+                float sum = 0.f;
+                for (int j = pi - P + 1; j < pi; ++j)
+                    sum += hb_ld(cache + v_base + ((size_t)pt[j / ps] * ps + j % ps) * (size_t)(G * vdim) + g * vdim + j2);
+                sum += hb_operand<T>(vs[j2]);
+                dst[dim + j2] = sum / (float)P;
+            }
+        }
     }
 }
 
@@ -1105,8 +1216,10 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             float* t = cur; cur = other; other = t;
         }
         const int n_in = hb_layer_in(L), n_mix = L.heads * L.vdim;
-        hb_layernorm(st, n, cur, ldx, nullptr, L.norm1, m->h, (long)W, W, c.eps);
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->h, W, (const T*)L.w_in, L.b_in, m->proj, n_in, n, n_in, W));
+        if (!(n == 1 && hb_try_ln_gemv<T>(st, HB_EPI_STORE, cur, ldx, nullptr, L.norm1, c.eps, (const T*)L.w_in, L.b_in, m->proj, n_in, W))) {
+            hb_layernorm(st, n, cur, ldx, nullptr, L.norm1, m->h, (long)W, W, c.eps);
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->h, W, (const T*)L.w_in, L.b_in, m->proj, n_in, n, n_in, W));
+        }
         const int vt = (L.vdim + 63) / 64;
         // dims per wave of the scans: the smallest of 16 / 32 / 64 that covers dim with at most 16 waves
         const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
@@ -1132,10 +1245,13 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             const int H = L.heads, G = L.kv_heads, QG = H / G;
             const long v_base = (long)c.max_pages * ps * G * L.dim;
             const int ppp = (ps - 1) / L.pool + 1;
+            const bool one_row_each = n == n_req;      // decode steps: every block a row closes was filled by earlier steps
             hipLaunchKernelGGL((k_hb_attn_prep<T>), dim3(n, H + G), dim3(64), 0, st, m->proj, (long)n_in, (T*)run.cache, L.inv_freq, io->pos,
-                               io->page, io->slot, H, G, L.dim, L.vdim, L.rot_dims, ps, v_base, c.eps);
-            hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)run.cache, run.pool, io->pos, io->row_req,
-                               io->page_table, io->pt_stride, G, L.dim, L.vdim, L.pool, ps, ppp, v_base);
+                               io->page, io->slot, H, G, L.dim, L.vdim, L.rot_dims, ps, v_base, c.eps, one_row_each ? run.pool : (float*)nullptr,
+                               io->row_req, io->page_table, io->pt_stride, L.pool, ppp);
+            if (!one_row_each)
+                hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)run.cache, run.pool, io->pos, io->row_req,
+                                   io->page_table, io->pt_stride, G, L.dim, L.vdim, L.pool, ps, ppp, v_base);
             const int split = 16 / QG >= 4 ? 4 : (16 / QG >= 1 ? 16 / QG : 1);      // up to 16 waves per block, at most 4 per head
             const int nwv2 = QG * split, dimp = (L.dim + 3) & ~3;
             const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (L.vdim + 2) * 4;
@@ -1153,16 +1269,21 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
         }
         VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix));
         if (L.ff > 0) {
-            hb_layernorm(st, n, cur, ldx, nullptr, L.norm2, m->h, (long)W, W, c.eps);
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
+            if (!(n == 1 && hb_try_ln_gemv<T>(st, HB_EPI_GELU, cur, ldx, nullptr, L.norm2, c.eps, (const T*)L.w_up, nullptr, m->ff, L.ff, W))) {
+                hb_layernorm(st, n, cur, ldx, nullptr, L.norm2, m->h, (long)W, W, c.eps);
+                VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
+            }
             VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff, L.ff, (const T*)L.w_down, nullptr, cur, ldx, n, W, L.ff));
         }
         if (io->trace)
             hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
     }
     if (n_out > 0) {
-        hb_layernorm(st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, (long)W, W, c.eps);
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits, c.vocab, n_out, c.vocab, W));
+        if (!(n_out == 1 && hb_try_ln_gemv<T>(st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, c.eps, (const T*)m->w.head, nullptr,
+                                              io->logits, c.vocab, W))) {
+            hb_layernorm(st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, (long)W, W, c.eps);
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits, c.vocab, n_out, c.vocab, W));
+        }
     }
     VOX_HIP(hipGetLastError());
     return VOX_OK;

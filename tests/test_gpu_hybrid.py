@@ -346,3 +346,41 @@ def test_top_k_sampling_through_the_scheduler():
             assert tok in top, (rid, tok, top)
             seq.append(tok)
     assert generate() == first
+
+
+def test_async_scheduling_generates_the_same_ids():
+    """The pipelined scheduler loop (a step is launched before the previous step's ids are read; a finished request gets one surplus
+    row that is dropped) generates the oracle's greedy ids too."""
+    from vox_serve_amd.model.sirodra import SirodraModel, config_from_dict
+    from vox_serve_amd.scheduler.base import Scheduler, encode_request
+    from vox_serve_amd.worker.base import ModelWorker
+    cfg = stack()
+    S = U.random_checkpoint(cfg, seed=71)
+    n_new = 9
+    model = SirodraModel("sirodra-test", S, config_from_dict(cfg), dtype=torch.float32, max_batch_size=4, page_size=8, max_num_pages=64,
+                         max_seq_len=512, max_prefill_tokens=64, state_slots=4, max_tokens=n_new)
+    worker = ModelWorker(model=model, max_batch_size=4, max_num_pages=64, page_size=8, greedy=True, prefill_chunk_tokens=20)
+    sched = Scheduler(worker, max_batch_size=4, async_scheduling=True)
+    prompts = {"p0": tokens(30, 64, 72), "p1": tokens(3, 64, 73), "p2": tokens(41, 64, 74)}
+    seen = {}
+    orig = sched._prepare_requests
+
+    def spy():
+        orig()
+        for r in sched.active_requests:
+            seen[r.request_id] = r
+    sched._prepare_requests = spy
+    try:
+        for rid, p in prompts.items():
+            sched.transport.requests.put(encode_request(rid, " ".join(map(str, p)), is_streaming=False))
+        sched.run_until_idle(max_steps=500)
+        assert set(seen) == set(prompts)
+        for rid, p in prompts.items():
+            seq = list(p)
+            for _ in range(n_new):
+                seq.append(int(HR.forward(cfg, S, seq)[-1].argmax()))
+            got = [int(t[0, 0]) for t in seen[rid].lm_output_tokens]
+            assert got[:n_new] == seq[len(p):], (rid, got, seq[len(p):])
+        assert worker.empty_pages.qsize() == 64 and worker.empty_state_slots.qsize() == 4
+    finally:
+        model.engine.close()

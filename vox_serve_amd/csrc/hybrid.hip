@@ -427,13 +427,13 @@ bool hb_try_ln_gemv(hipStream_t st, int epi, const float* X, long ldx, const int
     return true;
 }
 
-// 2..16 rows, bf16: one MFMA row tile; a block owns 16 output columns and its four waves take the 32-wide k-steps w, w + 4, ...
+// 2..16 rows, bf16: one MFMA row tile; a block owns 16 output columns and its eight waves take the 32-wide k-steps w, w + 8, ...
 // with both fragments straight from memory (the weight fragment is one 16-byte request per lane, the activation fragment two,
-// converted to bf16 in registers); the four partial tiles are added in wave order.  Needs K % 32 == 0.
+// converted to bf16 in registers); the eight partial tiles are added in wave order.  Needs K % 32 == 0.
 template <int EPI>
-__global__ __launch_bounds__(256) void k_hb_gemm_rows16(const float* A, long lda, const bf16_t* Wt, const float* bias, float* C, long ldc, int M,
+__global__ __launch_bounds__(512) void k_hb_gemm_rows16(const float* A, long lda, const bf16_t* Wt, const float* bias, float* C, long ldc, int M,
                                                         int N, int K) {
-    __shared__ float red[4][16][17];
+    __shared__ float red[8][16][17];
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int n0 = blockIdx.x * 16, col = lane & 15, kb = lane >> 4;
     const int nsteps = K >> 5;
@@ -442,12 +442,12 @@ __global__ __launch_bounds__(256) void k_hb_gemm_rows16(const float* A, long lda
     const float* arow = A + (size_t)(col < M ? col : M - 1) * lda + kb * 8;
     const bool rowok = col < M;
     constexpr int U = 8;
-    for (int s0 = wv; s0 < nsteps; s0 += 4 * U) {
+    for (int s0 = wv; s0 < nsteps; s0 += 8 * U) {
         uint4 wf[U];
         float4 a0[U], a1[U];
 #pragma unroll
         for (int u = 0; u < U; ++u) {
-            const int sidx = s0 + 4 * u;
+            const int sidx = s0 + 8 * u;
             const bool valid = sidx < nsteps;
             const int k = (valid ? sidx : s0) << 5;
             wf[u] = *(const uint4*)(wrow + k);
@@ -472,14 +472,14 @@ __global__ __launch_bounds__(256) void k_hb_gemm_rows16(const float* A, long lda
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
             const int row = kb * 4 + r;
-            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col], bz);
+            if (row < M) hb_epilogue<EPI>(C + (size_t)row * ldc + n0 + col, ((((((red[0][row][col] + red[1][row][col]) + red[2][row][col]) + red[3][row][col]) + red[4][row][col]) + red[5][row][col]) + red[6][row][col]) + red[7][row][col], bz);
         }
     }
 }
 template <int EPI>
 bool hb_try_rows16(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K) {
     if (M < 2 || M > 16 || (K & 31) || (lda & 3) || ((size_t)A & 15) || ((size_t)W & 15)) return false;
-    hipLaunchKernelGGL((k_hb_gemm_rows16<EPI>), dim3((N + 15) / 16), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+    hipLaunchKernelGGL((k_hb_gemm_rows16<EPI>), dim3((N + 15) / 16), dim3(512), 0, st, A, lda, W, bias, C, ldc, M, N, K);
     return true;
 }
 template <int EPI>

@@ -354,43 +354,98 @@ int vox_lm_prefill(vox_lm* m, void* stream, const vox_lm_io* io, const int32_t* 
                    int max_kvlen, const vox_sampling_config* sampling, uint64_t seed, int feedback);
 
 /* ---- hybrid-mixer LM engine ---------------------------------------------------------------------------------
- * A decoder whose layers mix tokens with a linear recurrence (HGRN2, mLSTM) or with sliding-window attention over a
- * paged cache that also keeps one mean key / value per block of older tokens; a contiguous range of layers may run
- * several times with the same weights (every run owns its cache or state).  Residual stream, norms, rotary angles,
- * scores, gates and recurrent states are fp32 in both dtypes; the dtype is the storage of the matrices and of the
- * K / V cache and the GEMM operand precision.  One step = a ragged set of rows (prompt portions next to single
- * decoded tokens); rows of a request are contiguous and ascending in position.                                     */
+ * A decoder whose layers mix tokens with a linear recurrence (HGRN2, mLSTM, a real-gated diagonal unit behind a short
+ * convolution, a matrix state with token shift and per-channel decay) or with attention over a paged cache (a sliding
+ * window that also keeps one mean key / value per block of older tokens, or plain causal attention with normed q / k /
+ * v); two mixers may run side by side on the same input; a contiguous range of layers may run several times with the
+ * same weights (every run owns its cache or state).  A layer is sequential (x += mixer(norm1 x); x += ff(norm2 x)) or
+ * parallel (x += mixer(norm1 x) + ff(norm2 x)); the feed-forward is dense or a routed mixture of experts.  Residual
+ * stream, norms, rotary angles, scores, routers, gates and recurrent states are fp32 in both dtypes; the dtype is the
+ * storage of the matrices and of the K / V cache and the GEMM operand precision.  One step = a ragged set of rows
+ * (prompt portions next to single decoded tokens); rows of a request are contiguous and ascending in position.      */
 typedef struct vox_hybrid vox_hybrid;
-enum { VOX_MIXER_HGRN2 = 0, VOX_MIXER_POOLED_WINDOW_ATTN = 1, VOX_MIXER_MLSTM = 2 };
+enum { VOX_MIXER_HGRN2 = 0, VOX_MIXER_POOLED_WINDOW_ATTN = 1, VOX_MIXER_MLSTM = 2, VOX_MIXER_RGLRU = 3, VOX_MIXER_CAUSAL_ATTN = 4,
+       VOX_MIXER_SHIFT_DECAY = 5 };
 enum { VOX_HYBRID_BF16 = 0, VOX_HYBRID_F32 = 1 };
+enum { VOX_NORM_LAYER = 0 /* weight-only layer norm */, VOX_NORM_RMS_GROUPS = 1 /* RMS norm over norm_groups equal slices */ };
+enum { VOX_BLOCK_SEQUENTIAL = 0, VOX_BLOCK_PARALLEL = 1 };
+/* Routed feed-forward.  Router logits z = router . h in fp32; s = softmax(z) over experts + identity outputs; the `top`
+ * largest of s + correction are chosen; their weights are s / (sum of the chosen s + 1e-20).  Expert e < experts:
+ * g = min(gate_e h, limit), u = clamp(up_e h, -limit, limit), y = g * sigmoid(act_alpha * g) * (u + 1), output down_e y.
+ * The last `identity` router outputs return h itself.  A shared expert of the same form (shared_ff > 0) runs for every row. */
+typedef struct {
+    int32_t experts, identity, top, ff, shared_ff;
+    float limit, shared_limit, act_alpha;
+    const float* router;          /* [experts + identity, width] fp32 */
+    const float* correction;      /* [experts + identity] fp32 or NULL */
+    const void* w_gate_up;        /* [experts][2*ff][width]: gate rows, then up rows; engine dtype */
+    const void* w_down;           /* [experts][width][ff] */
+    const void* shared_gate_up;   /* [2*shared_ff][width] */
+    const void* shared_down;      /* [width][shared_ff] */
+} vox_hybrid_moe;
 typedef struct {
     int32_t kind, heads, kv_heads, dim, vdim;
     int32_t window, pool, rot_dims;       /* attention: visible tokens, tokens per pooled block, rotated dims per head */
     float scale, gate_cap;                /* attention score scale; mLSTM soft cap of the gate pre-activations */
-    int32_t ff;                           /* feed-forward width, 0 = the layer has none */
+    int32_t ff;                           /* dense feed-forward width, 0 = none (a routed one hangs on `moe`) */
     const float *norm1, *norm2;           /* [width] fp32 */
     /* fused input projection, rows in this order:
-     *   HGRN2      q (heads*dim) | forget (heads*dim) | v (heads*vdim)
-     *   attention  q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim) | output gate (heads)
-     *   mLSTM      q (heads*dim) | k (heads*dim) | v (heads*vdim) | output gate (heads*vdim) | input gate (heads) | forget gate (heads) */
+     *   HGRN2         q (heads*dim) | forget (heads*dim) | v (heads*vdim)
+     *   pooled attn   q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim) | output gate (heads)
+     *   mLSTM         q (heads*dim) | k (heads*dim) | v (heads*vdim) | output gate (heads*vdim) | input gate (heads) | forget gate (heads)
+     *   RGLRU         gated branch (C) | recurrent branch (C), C = heads*dim channels in `heads` blocks of dim (= vdim)
+     *   causal attn   q (heads*dim) | k (kv_heads*dim) | v (kv_heads*vdim)
+     *   shift-decay   r | k | v | g (heads*dim each, dim = vdim) | decay bottleneck (lora); each of the five reads its own token-shift mix */
     const void* w_in;                     /* [n_in, width] engine dtype */
     const float* b_in;                    /* [n_in] fp32 or NULL */
     const void* w_out;                    /* [width, heads*vdim] */
     const float* lower;                   /* HGRN2: lower bound of the forget gate [heads*dim] */
-    const float* head_norm;               /* HGRN2: [vdim] shared by heads; mLSTM: [heads*vdim] */
-    const float* inv_freq;                /* attention: rotary frequencies [rot_dims/2] (scaling already applied) */
+    const float* head_norm;               /* HGRN2: [vdim] shared by heads; mLSTM, shift-decay: [heads*vdim] */
+    const float* inv_freq;                /* pooled attention: rotary frequencies [rot_dims/2] (scaling already applied) */
     const void *w_up, *w_down;            /* [ff, width], [width, ff] */
+    int32_t block;                        /* VOX_BLOCK_* */
+    int32_t sibling;                      /* -1, or the index of a layer record whose mixer runs beside this one on the same normed
+                                             input and joins the same sum (its own norms, block and feed-forward are not used) */
+    float out_scale;                      /* the mixer's output is multiplied by this before it joins the sum */
+    /* causal attention: RMS-norm weights of q and k [dim] shared by heads (NULL: unit RMS); q is also multiplied by
+     * 1 + q_temp_coef * ln(floor((p + 1) / q_temp_every) + 1) at position p; v_unit_rms: each head's value is divided by its RMS */
+    const float *q_norm, *k_norm;
+    float q_temp_coef;
+    int32_t q_temp_every, v_unit_rms;
+    /* RGLRU: u = causal conv of the recurrent branch (conv_w [C][conv_taps], last tap = current token; conv_b [C]); per block
+     * r | i = sigmoid(w_gates[b] u_b + b_gates[b]) (w_gates [heads][2*dim][dim]: rows of r, then of i); a = exp(-rec_scale * r *
+     * softplus(lam)); S <- a S + sqrt(1 - a^2) i u; mixer output = S * gelu_tanh(gated branch) */
+    int32_t conv_taps;
+    float rec_scale;
+    const float *conv_w, *conv_b;
+    const void* w_gates;
+    const float *b_gates, *lam;
+    /* shift-decay: mix_s = h + (h_prev - h) * shift_mu[s], s = r, k, v, g, w; decay = exp(-exp(w_decay2 tanh(bottleneck) + decay0));
+     * o = (S + diag(bonus) k v^T)^T r; S <- diag(decay) S + k v^T; then unit RMS per head * head_norm * silu(g) */
+    int32_t lora;
+    const float* shift_mu;                /* [5][width] fp32 */
+    const void* w_decay2;                 /* [heads*dim, lora] engine dtype */
+    const float *decay0, *bonus;          /* [heads*dim] fp32 each */
+    const vox_hybrid_moe* moe;            /* routed feed-forward or NULL */
 } vox_hybrid_layer;
 typedef struct {
     int32_t layer;       /* index into layers */
     int32_t loop_in;     /* 1: x <- loop_in [x; x0] before this run */
     void* cache;         /* attention: K [max_pages*page_size][kv_heads*dim] then V [max_pages*page_size][kv_heads*vdim], engine dtype */
-    float* pool;         /* attention: [max_pages][(page_size-1)/pool+1][kv_heads][dim+vdim] */
-    float* state;        /* HGRN2: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1] */
+    float* pool;         /* pooled attention: [max_pages][(page_size-1)/pool+1][kv_heads][dim+vdim] */
+    /* HGRN2: [slots][heads][dim][vdim]; mLSTM: [slots][heads][dim*vdim + dim + 1]; RGLRU: [slots][conv_taps][C] (S, then the last
+     * conv_taps-1 inputs of the convolution, oldest first); shift-decay: [slots][heads*dim*dim + width] (S, then the previous
+     * token's normed input) */
+    float* state;
+    void* side_cache;    /* the same three for the layer's sibling mixer */
+    float* side_pool;
+    float* side_state;
 } vox_hybrid_run;
 typedef struct {
     int32_t width, vocab, n_layers, n_runs, dtype, page_size, max_rows, max_batch, max_out, max_pages, max_seq_len;
     float eps;
+    int32_t norm_kind, norm_groups;       /* VOX_NORM_*; slices of the grouped RMS norm (>= 1) */
+    float embed_scale;                    /* x0 = embedding[id] * embed_scale */
 } vox_hybrid_config;
 typedef struct {
     const vox_hybrid_layer* layers;

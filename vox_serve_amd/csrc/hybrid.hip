@@ -1,6 +1,9 @@
-// Hybrid-mixer LM engine: a decoder whose layers mix tokens either with a linear recurrence (HGRN2, mLSTM) or with
-// sliding-window attention over a paged cache that also keeps one mean key / value per block of older tokens.  A contiguous
-// range of layers may run several times with the same weights; every run owns its cache or recurrent state.
+// Hybrid-mixer LM engine: a decoder whose layers mix tokens either with a linear recurrence (HGRN2, mLSTM, a real-gated diagonal
+// unit behind a short convolution, a matrix state with token shift and per-channel decay) or with attention over a paged cache
+// (a sliding window that also keeps one mean key / value per block of older tokens, or plain causal attention with normed
+// q / k / v).  Two mixers may run side by side on one input; a layer is sequential or parallel; its feed-forward is dense or a
+// routed mixture of experts.  A contiguous range of layers may run several times with the same weights; every run owns its
+// cache or recurrent state.
 //
 // Numeric rule of this engine: the residual stream, norms, rotary angles, attention scores / softmax, gates, decays and every
 // recurrent state are fp32.  The engine's dtype (bf16 or fp32) is the storage of the large matrices, of the K / V cache and of
@@ -41,22 +44,35 @@ template <typename T> __device__ __forceinline__ float hb_operand(float v);
 template <> __device__ __forceinline__ float hb_operand<float>(float v) { return v; }
 template <> __device__ __forceinline__ float hb_operand<bf16_t>(float v) { return bfround(v); }
 
-enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2 };
+enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2, HB_EPI_TANH = 3 };
 template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float acc, float bias) {
     float v = acc + bias;
     if (EPI == HB_EPI_GELU) v = 0.5f * v * (1.0f + erff(v * 0.70710678118654752440f));
+    if (EPI == HB_EPI_TANH) v = tanhf(v);
     if (EPI == HB_EPI_RESID) v = *c + v;
     *c = v;
 }
+__device__ __forceinline__ float hb_gelu_tanh(float z) {
+    return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
+}
+// A tile GEMM over a gathered subset of rows (routed experts): block z multiplies the rows list[z*cap + 0 .. count[z]) with the
+// z-th matrix (w_stride elements apart); the A row of list entry v is v / a_div, its C row is v.  count == NULL: plain GEMM.
+struct hb_rowmap {
+    const int* count;
+    const int* list;
+    int cap, a_div;
+    long w_stride;
+};
 
 // ---- embedding gather: x[row] = table[id]; the second half of both residual buffers keeps the embedding output ----------
 template <typename T>
-__global__ __launch_bounds__(256) void k_hb_embed(const T* table, const int* ids, int id_stride, float* xa, float* xb, int W, int vocab) {
+__global__ __launch_bounds__(256) void k_hb_embed(const T* table, const int* ids, int id_stride, float* xa, float* xb, int W, int vocab,
+                                                  float scale) {
     const int row = blockIdx.x;
     int id = ids[(size_t)row * id_stride];
     id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
     for (int i = threadIdx.x; i < W; i += 256) {
-        const float v = hb_ld(table + (size_t)id * W + i);
+        const float v = hb_ld(table + (size_t)id * W + i) * scale;
         xa[(size_t)row * 2 * W + i] = v;
         xa[(size_t)row * 2 * W + W + i] = v;
         xb[(size_t)row * 2 * W + W + i] = v;
@@ -124,17 +140,46 @@ static void hb_layernorm(hipStream_t st, int n, const float* x, long ldx, const 
     else hipLaunchKernelGGL(k_hb_layernorm<0>, dim3(n), dim3(256), 0, st, x, ldx, rows, w, y, ldy, W, eps);
 }
 
+// ---- RMS norm over `groups` equal consecutive slices of the row, fp32; optional row gather; one or two weights --------------
+// Every slice is divided by its own sqrt(mean square + eps); y1 = that * w1 and (w2 != NULL) y2 = that * w2: the two norms of a
+// parallel layer share their statistics.  One wave per slice (waves take slices w, w + 4, ...): lane-strided sum of squares, then
+// a butterfly — an order fixed by the slice length.
+__global__ __launch_bounds__(256) void k_hb_rms_groups(const float* x, long ldx, const int* rows, const float* w1, float* y1, const float* w2,
+                                                       float* y2, long ldy, int W, int groups, float eps) {
+    const int r = blockIdx.x, src = rows ? rows[r] : r, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    const int Wg = W / groups;
+    for (int g = wv; g < groups; g += 4) {
+        const float* xr = x + (size_t)src * ldx + (size_t)g * Wg;
+        float ss = 0.f;
+        for (int i = lane; i < Wg; i += 64) ss = fmaf(xr[i], xr[i], ss);
+        ss = hb_wave_sum(ss);
+        const float inv = 1.0f / sqrtf(ss / (float)Wg + eps);
+        for (int i = lane; i < Wg; i += 64) {
+            const float v = xr[i] * inv;
+            y1[(size_t)r * ldy + g * Wg + i] = v * w1[g * Wg + i];
+            if (w2) y2[(size_t)r * ldy + g * Wg + i] = v * w2[g * Wg + i];
+        }
+    }
+}
+
 // ---- GEMM  C[M,N] (+)= A[M,K] . W[N,K]^T + bias ---------------------------------------------------------------------------
 // bf16: both operands staged in LDS as bf16 (activations rounded once), v_mfma_f32_16x16x32_bf16; four waves, 64 output columns
 // per block, BM = 64 (2 x 2 tiles per wave) or BM = 16 (one tile per wave).  Every edge (M, N, K) is guarded at the LDS fill.
 template <int BM, int EPI>
 __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, const bf16_t* Wt, const float* bias, float* C, long ldc, int M,
-                                                      int N, int K) {
+                                                      int N, int K, hb_rowmap rm) {
     constexpr int BK = 64, LD = BK + 8;
     __shared__ __attribute__((aligned(16))) bf16_t As[BM * LD];
     __shared__ __attribute__((aligned(16))) bf16_t Ws[64 * LD];
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
+    const int* lst = nullptr;
+    if (rm.count) {
+        M = rm.count[blockIdx.z];
+        if (m0 >= M) return;
+        lst = rm.list + (size_t)blockIdx.z * rm.cap;
+        Wt += (size_t)blockIdx.z * rm.w_stride;
+    }
     constexpr int MT = BM == 64 ? 2 : 1, NT = BM == 64 ? 2 : 1;
     const int mt0 = BM == 64 ? (wv >> 1) * 2 : 0, nt0 = BM == 64 ? (wv & 1) * 2 : wv;
     hb_f32x4 acc[MT][NT];
@@ -151,7 +196,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
             const int gm = m0 + r, gk = k0 + c;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
             if (gm < M) {
-                const float* p = A + (size_t)gm * lda + gk;
+                const float* p = A + (size_t)(lst ? lst[gm] / rm.a_div : gm) * lda + gk;
                 if (a_vec && gk + 3 < K) v = *(const float4*)p;
                 else {
                     if (gk < K) v.x = p[0];
@@ -216,7 +261,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int gm = m0 + (mt0 + i) * 16 + (lane >> 4) * 4 + r;
-                if (gm < M) hb_epilogue<EPI>(C + (size_t)gm * ldc + gn, acc[i][j][r], b);
+                if (gm < M) hb_epilogue<EPI>(C + (size_t)(lst ? lst[gm] : gm) * ldc + gn, acc[i][j][r], b);
             }
         }
 }
@@ -224,12 +269,22 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
 // fp32: LDS-tiled FMA, 64 output columns per block, BM = 64 (4 x 4 per thread) or 16 (1 x 4 per thread); k ascending per element.
 template <int BM, int EPI>
 __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, const float* Wt, const float* bias, float* C, long ldc, int M,
-                                                     int N, int K) {
+                                                     int N, int K, hb_rowmap rm) {
     constexpr int BK = 16, RM = BM / 16;
     __shared__ float As[BK][BM + 4];
     __shared__ float Ws[BK][64 + 4];
+    __shared__ int arow[BM];
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
+    const int* lst = nullptr;
+    if (rm.count) {
+        M = rm.count[blockIdx.z];
+        if (m0 >= M) return;
+        lst = rm.list + (size_t)blockIdx.z * rm.cap;
+        Wt += (size_t)blockIdx.z * rm.w_stride;
+    }
+    for (int r = tid; r < BM; r += 256) arow[r] = m0 + r < M ? (lst ? lst[m0 + r] : m0 + r) : -1;
+    __syncthreads();
     float acc[RM][4];
 #pragma unroll
     for (int i = 0; i < RM; ++i)
@@ -239,7 +294,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
         for (int idx = tid; idx < BM * BK; idx += 256) {
             const int r = idx / BK, c = idx % BK;
             const int gm = m0 + r, gk = k0 + c;
-            As[c][r] = (gm < M && gk < K) ? A[(size_t)gm * lda + gk] : 0.f;
+            As[c][r] = (gm < M && gk < K) ? A[(size_t)(lst ? arow[r] / rm.a_div : gm) * lda + gk] : 0.f;
         }
         for (int idx = tid; idx < 64 * BK; idx += 256) {
             const int r = idx / BK, c = idx % BK;
@@ -268,7 +323,7 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const int gn = n0 + tx * 4 + j;
-            if (gn < N) hb_epilogue<EPI>(C + (size_t)gm * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f);
+            if (gn < N) hb_epilogue<EPI>(C + (size_t)arow[ty * RM + i] * ldc + gn, acc[i][j], bias ? bias[gn] : 0.f);
         }
     }
 }
@@ -488,16 +543,19 @@ bool hb_try_rows16(hipStream_t, const float*, long, const float*, const float*, 
 template <typename T, int EPI>
 int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K);
 
+// rm.count != NULL: `groups` gathered GEMMs of at most M rows each in one launch (see hb_rowmap)
 template <int EPI>
-int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K) {
-    if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_bf16<16, EPI>), dim3((N + 63) / 64, 1), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
-    else hipLaunchKernelGGL((k_hb_gemm_bf16<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K,
+                  hb_rowmap rm = hb_rowmap{nullptr, nullptr, 0, 1, 0}, int groups = 1) {
+    if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_bf16<16, EPI>), dim3((N + 63) / 64, 1, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
+    else hipLaunchKernelGGL((k_hb_gemm_bf16<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     return VOX_OK;
 }
 template <int EPI>
-int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const float* W, const float* bias, float* C, long ldc, int M, int N, int K) {
-    if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_f32<16, EPI>), dim3((N + 63) / 64, 1), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
-    else hipLaunchKernelGGL((k_hb_gemm_f32<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const float* W, const float* bias, float* C, long ldc, int M, int N, int K,
+                  hb_rowmap rm = hb_rowmap{nullptr, nullptr, 0, 1, 0}, int groups = 1) {
+    if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_f32<16, EPI>), dim3((N + 63) / 64, 1, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
+    else hipLaunchKernelGGL((k_hb_gemm_f32<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     return VOX_OK;
 }
 template <typename T, int EPI>
@@ -524,6 +582,7 @@ template <typename T>
 int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
     if (epi == HB_EPI_GELU) return hb_gemm_epi<T, HB_EPI_GELU>(st, A, lda, W, bias, C, ldc, M, N, K);
     if (epi == HB_EPI_RESID) return hb_gemm_epi<T, HB_EPI_RESID>(st, A, lda, W, bias, C, ldc, M, N, K);
+    if (epi == HB_EPI_TANH) return hb_gemm_epi<T, HB_EPI_TANH>(st, A, lda, W, bias, C, ldc, M, N, K);
     return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K);
 }
 
@@ -699,9 +758,10 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_mlstm_scan(const 
 }
 
 // per (row, head): o / rms(o) over vdim, times a weight (per_head_w: indexed over all heads, else shared [vdim]), times
-// sigmoid(gate) when gate_off >= 0 (gate = proj[row][gate_off + h*vdim + j]).  In place.
+// a gate (gate_mode 1: sigmoid(g), 2: g * sigmoid(g); g = proj[row][gate_off + h*vdim + j]), times out_scale.  In place.
+enum { HB_GATE_NONE = 0, HB_GATE_SIGMOID = 1, HB_GATE_SILU = 2 };
 __global__ __launch_bounds__(64) void k_hb_head_norm(float* o, long ldo, const float* w, int per_head_w, const float* proj, long ldp, int gate_off,
-                                                     int vdim, float eps) {
+                                                     int gate_mode, int vdim, float eps, float out_scale) {
     const int row = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     float* p = o + (size_t)row * ldo + (size_t)h * vdim;
     float ss = 0.f;
@@ -710,18 +770,194 @@ __global__ __launch_bounds__(64) void k_hb_head_norm(float* o, long ldo, const f
     const float inv = 1.0f / sqrtf(ss / (float)vdim + eps);
     for (int j = lane; j < vdim; j += 64) {
         float v = p[j] * inv * w[per_head_w ? h * vdim + j : j];
-        if (gate_off >= 0) v *= hb_sigmoid(proj[(size_t)row * ldp + gate_off + h * vdim + j]);
-        p[j] = v;
+        if (gate_mode != HB_GATE_NONE) {
+            const float g = proj[(size_t)row * ldp + gate_off + h * vdim + j];
+            v *= gate_mode == HB_GATE_SIGMOID ? hb_sigmoid(g) : g * hb_sigmoid(g);
+        }
+        p[j] = v * out_scale;
+    }
+}
+
+// ---- real-gated linear recurrent unit behind a short causal convolution ------------------------------------------------------
+// proj row = [gated branch y (C) | recurrent branch x (C) | u = conv(x) (C) | gate pre-activations, per block r (bs) then i (bs)].
+// State of a slot: [taps][C]: row 0 the recurrent state, rows 1 .. taps-1 the last taps-1 inputs of the convolution, oldest first.
+// u[row][c] = conv_b[c] + sum_j conv_w[c][j] * x[position - (taps-1-j)][c]; inputs before the step's first row come from the slot,
+// inputs before the sequence are zero (so a portion that starts at position 0 never reads the slot).
+__global__ __launch_bounds__(256) void k_hb_conv_causal(float* proj, long ldp, const float* cw, const float* cb, const float* state,
+                                                        const int* pos, const int* row_req, const int* req_rows, const int* req_state, int C,
+                                                        int taps) {
+    const int row = blockIdx.x, c = blockIdx.y * 256 + threadIdx.x;
+    if (c >= C) return;
+    const int r = row_req[row], rs = req_rows[r], p = pos[row], p0 = pos[rs];
+    const float* hist = state + (size_t)req_state[r] * taps * C + C;
+    float acc = cb ? cb[c] : 0.f;
+    for (int j = 0; j < taps; ++j) {
+        const int back = taps - 1 - j, q = p - back;
+        if (q < 0) continue;
+        const float v = row - back >= rs ? proj[(size_t)(row - back) * ldp + C + c] : hist[(size_t)(q - (p0 - (taps - 1))) * C + c];
+        acc = fmaf(cw[(size_t)c * taps + j], v, acc);
+    }
+    proj[(size_t)row * ldp + 2 * C + c] = acc;
+}
+// One thread per (request, channel): walks the portion's tokens in order.  Per token: r, i = sigmoid(gate pre-activations),
+// a = exp(-rec_scale * r * softplus(lam)), S <- a S + sqrt(1 - a^2) (i u), out = S * gelu_tanh(y) * out_scale.  The inputs of 8 tokens
+// are fetched and their gates evaluated before the 8 dependent updates.  At the end the slot's convolution history is shifted:
+// entry i <- the input at position (end - (taps-1) + i), from this step's rows or from the old history (ascending i, in place).
+__global__ __launch_bounds__(64) void k_hb_rglru_scan(const float* proj, long ldp, float* out, long ldo, const float* lam, float* state,
+                                                      const int* req_rows, const int* req_state, const int* pos, int C, int bs, int taps,
+                                                      float rec_scale, float out_scale) {
+    const int r = blockIdx.x, c = blockIdx.y * 64 + threadIdx.x;
+    if (c >= C) return;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    float* st = state + (size_t)req_state[r] * taps * C;
+    const int p0 = pos[rs];
+    float S = p0 == 0 ? 0.f : st[c];
+    const float lv = lam[c];
+    const float sp = lv > 20.f ? lv : log1pf(expf(lv));
+    const int blk = c / bs, j = c - blk * bs;
+    const size_t off_r = (size_t)3 * C + (size_t)blk * 2 * bs + j, off_i = off_r + bs;
+    for (int t0 = rs; t0 < re; t0 += 8) {
+        float a[8], b[8], y[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int t = t0 + k < re ? t0 + k : re - 1;
+            const float* pr = proj + (size_t)t * ldp;
+            const float rg = hb_sigmoid(pr[off_r]), ig = hb_sigmoid(pr[off_i]);
+            a[k] = expf(-rec_scale * rg * sp);
+            b[k] = sqrtf(1.0f - a[k] * a[k]) * (ig * pr[2 * C + c]);
+            y[k] = hb_gelu_tanh(pr[c]);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k)
+            if (t0 + k < re) {
+                S = a[k] * S + b[k];
+                out[(size_t)(t0 + k) * ldo + c] = S * y[k] * out_scale;
+            }
+    }
+    st[c] = S;
+    const int n = re - rs;
+    for (int i = 0; i < taps - 1; ++i) {
+        const int q = p0 + n - (taps - 1) + i;
+        float v = 0.f;
+        if (q >= p0) v = proj[(size_t)(rs + q - p0) * ldp + C + c];
+        else if (q >= 0) v = st[(size_t)(1 + i + n) * C + c];
+        st[(size_t)(1 + i) * C + c] = v;
+    }
+}
+
+// ---- matrix-state recurrence with token shift and a data-dependent decay per key channel ------------------------------------
+// mixes[s][row] = h[row] + (h_prev - h[row]) * mu[s], s < 5; h_prev is the previous row of the request, or what the slot keeps
+// behind its matrix state (the previous step's last normed input), or zero at position 0.
+__global__ __launch_bounds__(256) void k_hb_shift_mix(const float* h, long ldh, const float* mu, float* mixes, long rows_stride, const float* state,
+                                                      long per_slot, long prev_off, const int* pos, const int* row_req, const int* req_rows,
+                                                      const int* req_state, int W) {
+    const int row = blockIdx.x;
+    const int r = row_req[row], rs = req_rows[r];
+    const float* prev = row > rs ? h + (size_t)(row - 1) * ldh : (pos[row] == 0 ? nullptr : state + (size_t)req_state[r] * per_slot + prev_off);
+    for (int i = threadIdx.x; i < W; i += 256) {
+        const float x = h[(size_t)row * ldh + i], d = (prev ? prev[i] : 0.f) - x;
+#pragma unroll
+        for (int s2 = 0; s2 < 5; ++s2) mixes[(size_t)s2 * rows_stride + (size_t)row * W + i] = x + d * mu[(size_t)s2 * W + i];
+    }
+}
+// proj row = [r | k | v | g (H*dim each) | decay bottleneck (lora) | decay pre-activation d (H*dim)]; decay = exp(-exp(d)).
+// Block = (request, head, 64 value columns); wave w keeps DPW key dims of the state in registers for the whole portion.  Per
+// token: o = sum_i (S_i + bonus_i k_i v) r_i, then S_i <- decay_i S_i + k_i v; the waves' partial outputs are added in wave order.
+// Block (r, 0, 0) finally stores the request's last normed input behind the matrix state (the next step's h_prev).
+template <int DPW>
+__global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(const float* proj, long ldp, float* out, long ldo, const float* bonus,
+                                                                                float* state, long per_slot, const float* h, long ldh, int W,
+                                                                                const int* req_rows, const int* req_state, const int* pos,
+                                                                                int H, int dim, int lora, int TT) {
+    extern __shared__ float sm[];
+    const int nw = blockDim.x >> 6, dpad = nw * DPW;
+    float* rsm = sm;                       // [TT][dpad]
+    float* ksm = rsm + TT * dpad;          // [TT][dpad]
+    float* wsm = ksm + TT * dpad;          // [TT][dpad]
+    float* vsm = wsm + TT * dpad;          // [TT][64]
+    float* part = vsm + TT * 64;           // [2][nw][64]
+    const int r = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.z * 64 + lane;
+    const int d0 = w * DPW;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const bool ok = c < dim, fresh = pos[rs] == 0;
+    float* slot = state + (size_t)req_state[r] * per_slot;
+    float* St = slot + (size_t)hd * dim * dim;
+    float S[DPW], u[DPW];
+#pragma unroll
+    for (int i = 0; i < DPW; ++i) {
+        S[i] = (ok && !fresh && d0 + i < dim) ? St[(size_t)(d0 + i) * dim + c] : 0.f;
+        u[i] = d0 + i < dim ? bonus[hd * dim + d0 + i] : 0.f;
+    }
+    const int HD = H * dim, off_d = 4 * HD + lora;
+    int flip = 0;
+    for (int t0 = rs; t0 < re; t0 += TT) {
+        const int nt = re - t0 < TT ? re - t0 : TT;
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < nt * dpad; idx += blockDim.x) {
+            const int tt = idx / dpad, d = idx - tt * dpad;
+            float rv = 0.f, kv = 0.f, wv = 0.f;
+            if (d < dim) {
+                const float* p = proj + (size_t)(t0 + tt) * ldp + hd * dim + d;
+                rv = p[0];
+                kv = p[HD];
+                wv = expf(-expf(p[off_d]));
+            }
+            rsm[idx] = rv; ksm[idx] = kv; wsm[idx] = wv;
+        }
+        for (int idx = threadIdx.x; idx < nt * 64; idx += blockDim.x) {
+            const int tt = idx >> 6, cc = blockIdx.z * 64 + (idx & 63);
+            vsm[idx] = cc < dim ? proj[(size_t)(t0 + tt) * ldp + 2 * HD + hd * dim + cc] : 0.f;
+        }
+        __syncthreads();
+        for (int tt = 0; tt < nt; ++tt) {
+            const float v = vsm[tt * 64 + lane];
+            const float* rt = rsm + tt * dpad + d0;
+            const float* kt = ksm + tt * dpad + d0;
+            const float* wt = wsm + tt * dpad + d0;
+            float o = 0.f;
+#pragma unroll
+            for (int i = 0; i < DPW; ++i) {
+                const float kv = kt[i] * v;
+                o = fmaf(S[i] + u[i] * kv, rt[i], o);
+                S[i] = wt[i] * S[i] + kv;
+            }
+            float* pt = part + flip * nw * 64;
+            pt[w * 64 + lane] = o;
+            __syncthreads();
+            if (w == 0 && ok) {
+                float sum = pt[lane];
+                for (int k = 1; k < nw; ++k) sum += pt[k * 64 + lane];
+                out[(size_t)(t0 + tt) * ldo + hd * dim + c] = sum;
+            }
+            flip ^= 1;
+        }
+    }
+    if (ok)
+#pragma unroll
+        for (int i = 0; i < DPW; ++i)
+            if (d0 + i < dim) St[(size_t)(d0 + i) * dim + c] = S[i];
+    if (hd == 0 && blockIdx.z == 0) {
+        float* prev = slot + (size_t)H * dim * dim;
+        for (int i = threadIdx.x; i < W; i += blockDim.x) prev[i] = h[(size_t)(re - 1) * ldh + i];
     }
 }
 
 // ---- attention: rotary (interleaved pairs, first `rot` dims) + unit RMS on q and k, K / V into the paged cache -----------
 // proj row = [q (H*dim) | k (G*dim) | v (G*vdim) | gate (H)].  Cache of one run: K [pages*ps][G*dim] then V [pages*ps][G*vdim].
+// Options of the plain causal form: a weight on the normed q / k (shared by heads), a query temperature
+// 1 + coef * ln(floor((p + 1) / every) + 1) at position p (coef 0: none), values divided by their RMS over vdim before they are cached.
 #define HB_MAX_DPL 8   // dims per lane: dim <= 512
+struct hb_qkv_opts {
+    const float *q_norm, *k_norm;
+    float temp_coef;
+    int temp_every, v_unit;
+};
 template <typename T>
 __global__ __launch_bounds__(64) void k_hb_attn_prep(float* proj, long ldp, T* cache, const float* inv_freq, const int* pos, const int* page,
                                                      const int* slot, int H, int G, int dim, int vdim, int rot, int ps, long v_base, float eps,
-                                                     float* pool, const int* row_req, const int* ptab, int pts, int P, int ppp) {
+                                                     float* pool, const int* row_req, const int* ptab, int pts, int P, int ppp, hb_qkv_opts op) {
     const int row = blockIdx.x, hb = blockIdx.y, lane = threadIdx.x;
     const bool is_q = hb < H;
     const int g = hb - H;
@@ -747,20 +983,30 @@ __global__ __launch_bounds__(64) void k_hb_attn_prep(float* proj, long ldp, T* c
         }
     }
     ss = hb_wave_sum(ss);
-    const float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+    float inv = 1.0f / sqrtf(ss / (float)dim + eps);
+    const float* nw = is_q ? op.q_norm : op.k_norm;
+    const float temp = is_q && op.temp_coef != 0.f ? 1.0f + op.temp_coef * logf((float)((pos[row] + 1) / op.temp_every) + 1.0f) : 1.0f;
     const size_t tok = (size_t)page[row] * ps + slot[row];
     // every lane has read its inputs (both pair members) before anyone overwrites: one wave, the reduction above is the fence
 #pragma unroll
     for (int e = 0; e < HB_MAX_DPL; ++e) {
         const int d = lane + e * 64;
         if (d < dim) {
-            if (is_q) src[d] = y[e] * inv;
-            else hb_st(cache + tok * (size_t)(G * dim) + g * dim + d, y[e] * inv);
+            float o = y[e] * inv;
+            if (nw) o *= nw[d];
+            if (is_q) src[d] = o * temp;
+            else hb_st(cache + tok * (size_t)(G * dim) + g * dim + d, o);
         }
     }
     if (!is_q) {
         const float* vs = proj + (size_t)row * ldp + H * dim + G * dim + g * vdim;
-        for (int j = lane; j < vdim; j += 64) hb_st(cache + v_base + tok * (size_t)(G * vdim) + g * vdim + j, vs[j]);
+        float vinv = 1.0f;
+        if (op.v_unit) {
+            float vv = 0.f;
+            for (int j = lane; j < vdim; j += 64) vv = fmaf(vs[j], vs[j], vv);
+            vinv = 1.0f / sqrtf(hb_wave_sum(vv) / (float)vdim + eps);
+        }
+        for (int j = lane; j < vdim; j += 64) hb_st(cache + v_base + tok * (size_t)(G * vdim) + g * vdim + j, vs[j] * vinv);
         // steps with one row per request (pool != NULL): the pooled entry of a block this token closes, here instead of in a launch
         // of its own — the block's other tokens were cached by earlier steps; this row's own values enter as the cache rounds them,
         // last, which is k_hb_pool_update's arithmetic
@@ -869,7 +1115,7 @@ __device__ __forceinline__ float hb_dot_slices(const float* q, const bf16_t* k, 
 template <typename T>
 __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) void k_hb_attn(const float* proj, long ldp, const T* cache, const float* pool, float* out, long ldo, const int* pos,
                           const int* row_req, const int* ptab, int pts, int H, int G, int dim, int vdim, int window, int P, int ps, int ppp,
-                          long v_base, float scale, int split, int seg_chunks, float* part) {
+                          long v_base, float scale, int split, int seg_chunks, float* part, int gated, float out_scale) {
     extern __shared__ float sm[];
     const int QG = H / G, NWV = QG * split;
     const int dimp = (dim + 3) & ~3;
@@ -1104,7 +1350,7 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
             if (lane == 0) { dst[vdim] = mm; dst[vdim + 1] = lt; }
             return;
         }
-        const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
+        const float gate = (gated ? hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]) : 1.0f) * out_scale;
         for (int j = lane; j < vdim; j += 64) {
             float a = 0.f;
             for (int s2 = 0; s2 < split; ++s2) {
@@ -1118,7 +1364,8 @@ __global__ __launch_bounds__(1024) __attribute__((amdgpu_waves_per_eu(1, 4))) vo
 
 // few-row steps: the segments' partial results of a (row, head), merged in segment order; output gate applied here
 __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nseg_grid, const float* proj, long ldp, float* out, long ldo,
-                                                      const int* pos, int H, int G, int dim, int vdim, int window, int P, int seg_chunks) {
+                                                      const int* pos, int H, int G, int dim, int vdim, int window, int P, int seg_chunks, int gated,
+                                                      float out_scale) {
     const int row = blockIdx.x, hq = blockIdx.y, lane = threadIdx.x;
     const int p = pos[row];
     const int first = p - window + 1;
@@ -1129,11 +1376,171 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
     for (int s2 = 0; s2 < nseg; ++s2) mm = fmaxf(mm, src[(size_t)s2 * (vdim + 2) + vdim]);
     float lt = 0.f;
     for (int s2 = 0; s2 < nseg; ++s2) lt += src[(size_t)s2 * (vdim + 2) + vdim + 1] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
-    const float gate = hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]);
+    const float gate = (gated ? hb_sigmoid(proj[(size_t)row * ldp + H * dim + G * dim + G * vdim + hq]) : 1.0f) * out_scale;
     for (int j = lane; j < vdim; j += 64) {
         float a = 0.f;
         for (int s2 = 0; s2 < nseg; ++s2) a += src[(size_t)s2 * (vdim + 2) + j] * expf(src[(size_t)s2 * (vdim + 2) + vdim] - mm);
         out[(size_t)row * ldo + hq * vdim + j] = a / lt * gate;
+    }
+}
+
+// ---- routed feed-forward --------------------------------------------------------------------------------------------------
+// One wave per row: s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first index
+// wins a tie) in descending order; weights = their s / (sum + 1e-20).  sel[row*top + k] = router output index, wgt likewise.
+__global__ __launch_bounds__(64) void k_hb_moe_route(const float* z, const float* corr, int nE, int top, int* sel, float* wgt) {
+    extern __shared__ float sm[];
+    float* sc = sm;                    // [nE] scores
+    float* ch = sm + nE;               // [nE] choice values
+    int* pick = (int*)(sm + 2 * nE);   // [top]
+    const int row = blockIdx.x, lane = threadIdx.x;
+    const float* zr = z + (size_t)row * nE;
+    float mx = -INFINITY;
+    for (int i = lane; i < nE; i += 64) mx = fmaxf(mx, zr[i]);
+    mx = hb_wave_max(mx);
+    float sum = 0.f;
+    for (int i = lane; i < nE; i += 64) {
+        const float e = expf(zr[i] - mx);
+        sc[i] = e;
+        sum += e;
+    }
+    sum = hb_wave_sum(sum);
+    for (int i = lane; i < nE; i += 64) {
+        const float v = sc[i] / sum;
+        sc[i] = v;
+        ch[i] = v + (corr ? corr[i] : 0.f);
+    }
+    __syncthreads();
+    float wsum = 0.f;
+    for (int k = 0; k < top; ++k) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int i = lane; i < nE; i += 64) {
+            const float v = ch[i];
+            if (v > best || (v == best && i < at)) { best = v; at = i; }
+        }
+#pragma unroll
+        for (int o = 32; o >= 1; o >>= 1) {
+            const float ov = __shfl_xor(best, o, 64);
+            const int oi = __shfl_xor(at, o, 64);
+            if (ov > best || (ov == best && oi < at)) { best = ov; at = oi; }
+        }
+        if (at == 0x7fffffff) at = 0;
+        wsum += sc[at];
+        __syncthreads();
+        if (lane == 0) { pick[k] = at; ch[at] = -INFINITY; }
+        __syncthreads();
+    }
+    const float den = wsum + 1e-20f;
+    for (int k = lane; k < top; k += 64) {
+        sel[(size_t)row * top + k] = pick[k];
+        wgt[(size_t)row * top + k] = sc[pick[k]] / den;
+    }
+}
+// Block e lists the entries (row*top + k) routed to expert e, ascending: list[e*cap + 0 .. count[e]).
+__global__ __launch_bounds__(256) void k_hb_moe_group(const int* sel, int n_entries, int cap, int* list, int* count) {
+    __shared__ int wsum[4];
+    __shared__ int base;
+    const int e = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
+    if (threadIdx.x == 0) base = 0;
+    __syncthreads();
+    for (int i0 = 0; i0 < n_entries; i0 += 256) {
+        const int i = i0 + threadIdx.x;
+        const bool hit = i < n_entries && sel[i] == e;
+        const unsigned long long bal = __ballot(hit);
+        const int before = __popcll(bal & ((1ull << lane) - 1ull));
+        if (lane == 0) wsum[wv] = __popcll(bal);
+        __syncthreads();
+        int off = base;
+        for (int w = 0; w < wv; ++w) off += wsum[w];
+        if (hit) list[(size_t)e * cap + off + before] = i;
+        __syncthreads();
+        if (threadIdx.x == 0) base += wsum[0] + wsum[1] + wsum[2] + wsum[3];
+        __syncthreads();
+    }
+    if (threadIdx.x == 0) count[e] = base;
+}
+// y = g * sigmoid(alpha g) * (u + 1), g = min(gate, limit), u = clamp(up, -limit, limit); gu row = [gate (ff) | up (ff)].
+// sel != NULL: rows are routed entries, those of identity outputs (sel >= experts) are skipped.
+__global__ __launch_bounds__(256) void k_hb_glu_clamp(const float* gu, float* y, int ff, float limit, float alpha, const int* sel, int experts) {
+    const int row = blockIdx.x;
+    if (sel && sel[row] >= experts) return;
+    for (int j = blockIdx.y * 256 + threadIdx.x; j < ff; j += gridDim.y * 256) {
+        const float g = fminf(gu[(size_t)row * 2 * ff + j], limit);
+        const float u = fminf(fmaxf(gu[(size_t)row * 2 * ff + ff + j], -limit), limit);
+        y[(size_t)row * ff + j] = g * hb_sigmoid(alpha * g) * (u + 1.0f);
+    }
+}
+// Few-row steps: one routed entry per blockIdx.y, a wave per output column (the order of k_hb_gemv's sum).  A row = entry / a_div,
+// the matrix is the entry's expert's; entries of identity outputs are skipped.  GLU: the wave takes the gate row n and the up row
+// ff + n and stores the activated value (N = ff output columns); else a plain product with N columns.
+template <typename T, bool GLU>
+__global__ __launch_bounds__(256) void k_hb_moe_gemv(const float* A, long lda, int a_div, const T* Wt, long w_stride, const int* sel, int experts,
+                                                     float* C, long ldc, int N, int K, float limit, float alpha) {
+    const int entry = blockIdx.y, lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int e = sel[entry];
+    if (n >= N || e >= experts) return;
+    const float* xr = A + (size_t)(entry / a_div) * lda;
+    const T* w0 = Wt + (size_t)e * w_stride + (size_t)n * K;
+    const T* w1 = w0 + (size_t)N * K;
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    float a0 = 0.f, a1 = 0.f;
+    const bool vec = (K % CH == 0) && ((((size_t)Wt) & 15) == 0) && ((w_stride * sizeof(T)) % 16 == 0) && (lda % 4 == 0) && ((((size_t)A) & 15) == 0);
+    if (vec) {
+        for (int k = lane * CH; k < K; k += 64 * CH) {
+            float wa[CH], wb[CH];
+            if (sizeof(T) == 2) {
+                const uint4 u = *(const uint4*)(w0 + k);
+                wa[0] = bflo(u.x); wa[1] = bfhi(u.x); wa[2] = bflo(u.y); wa[3] = bfhi(u.y);
+                if (CH == 8) { wa[4] = bflo(u.z); wa[5] = bfhi(u.z); wa[6] = bflo(u.w); wa[7] = bfhi(u.w); }
+                if (GLU) {
+                    const uint4 u2 = *(const uint4*)(w1 + k);
+                    wb[0] = bflo(u2.x); wb[1] = bfhi(u2.x); wb[2] = bflo(u2.y); wb[3] = bfhi(u2.y);
+                    if (CH == 8) { wb[4] = bflo(u2.z); wb[5] = bfhi(u2.z); wb[6] = bflo(u2.w); wb[7] = bfhi(u2.w); }
+                }
+            } else {
+                const float4 u = *(const float4*)(w0 + k);
+                wa[0] = u.x; wa[1] = u.y; wa[2] = u.z; wa[3] = u.w;
+                if (GLU) {
+                    const float4 u2 = *(const float4*)(w1 + k);
+                    wb[0] = u2.x; wb[1] = u2.y; wb[2] = u2.z; wb[3] = u2.w;
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < CH; ++i) {
+                const float x = hb_operand<T>(xr[k + i]);
+                a0 = fmaf(wa[i], x, a0);
+                if (GLU) a1 = fmaf(wb[i], x, a1);
+            }
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) {
+            const float x = hb_operand<T>(xr[k]);
+            a0 = fmaf(hb_ld(w0 + k), x, a0);
+            if (GLU) a1 = fmaf(hb_ld(w1 + k), x, a1);
+        }
+    }
+    a0 = hb_wave_sum(a0);
+    if (GLU) a1 = hb_wave_sum(a1);
+    if (lane == 0) {
+        if (GLU) {
+            const float g = fminf(a0, limit), u = fminf(fmaxf(a1, -limit), limit);
+            C[(size_t)entry * ldc + n] = g * hb_sigmoid(alpha * g) * (u + 1.0f);
+        } else {
+            C[(size_t)entry * ldc + n] = a0;
+        }
+    }
+}
+// x[row] += sum_k wgt[row*top + k] * (identity output ? h[row] : expert_out[row*top + k]), k ascending
+__global__ __launch_bounds__(256) void k_hb_moe_combine(float* x, long ldx, const float* h, long ldh, const float* eo, const int* sel,
+                                                        const float* wgt, int top, int experts, int W) {
+    const int row = blockIdx.x;
+    for (int i = threadIdx.x; i < W; i += 256) {
+        float acc = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const size_t en = (size_t)row * top + k;
+            acc = fmaf(wgt[en], sel[en] >= experts ? h[(size_t)row * ldh + i] : eo[en * W + i], acc);
+        }
+        x[(size_t)row * ldx + i] += acc;
     }
 }
 
@@ -1183,30 +1590,201 @@ struct vox_hybrid {
     vox_ctx* ctx;
     vox_hybrid_config cfg;
     std::vector<vox_hybrid_layer> layers;
+    std::vector<vox_hybrid_moe> moes;      // copies of the layers' routed feed-forwards (layers[i].moe points into this)
     std::vector<vox_hybrid_run> runs;
     vox_hybrid_weights w;
-    float *xa = nullptr, *xb = nullptr, *h = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
+    float *xa = nullptr, *xb = nullptr, *h = nullptr, *h2 = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
+    float *shift = nullptr;                 // [5][max_rows][width]: token-shift mixes
+    float *moe_z = nullptr, *moe_wgt = nullptr, *moe_act = nullptr, *moe_out = nullptr;
+    int *moe_sel = nullptr, *moe_list = nullptr, *moe_count = nullptr;
     bf16_t* logits16 = nullptr;
     float* attn_ws = nullptr;
     size_t attn_ws_bytes = 0;
     int max_in = 0, max_mix = 0, max_ff = 0;
+    int max_ne = 0, max_top = 0, max_eff = 0, max_experts = 0;
+    bool any_shift = false;
 };
 
+static bool hb_is_attn(int kind) { return kind == VOX_MIXER_POOLED_WINDOW_ATTN || kind == VOX_MIXER_CAUSAL_ATTN; }
+// rows of the fused input projection
 static int hb_layer_in(const vox_hybrid_layer& L) {
     switch (L.kind) {
         case VOX_MIXER_HGRN2: return 2 * L.heads * L.dim + L.heads * L.vdim;
         case VOX_MIXER_POOLED_WINDOW_ATTN: return L.heads * L.dim + L.kv_heads * (L.dim + L.vdim) + L.heads;
         case VOX_MIXER_MLSTM: return 2 * L.heads * L.dim + 2 * L.heads * L.vdim + 2 * L.heads;
+        case VOX_MIXER_RGLRU: return 2 * L.heads * L.dim;
+        case VOX_MIXER_CAUSAL_ATTN: return L.heads * L.dim + L.kv_heads * (L.dim + L.vdim);
+        case VOX_MIXER_SHIFT_DECAY: return 4 * L.heads * L.dim + L.lora;
     }
     return -1;
+}
+// floats per row of the projection buffer: the projection's outputs and what the mixer derives from them
+static int hb_layer_proj(const vox_hybrid_layer& L) {
+    if (L.kind == VOX_MIXER_RGLRU) return 5 * L.heads * L.dim;                           // + conv output, 2 gates
+    if (L.kind == VOX_MIXER_SHIFT_DECAY) return 5 * L.heads * L.dim + L.lora;            // + decay pre-activation
+    return hb_layer_in(L);
+}
+
+static void hb_norm(const vox_hybrid* m, hipStream_t st, int n, const float* x, long ldx, const int* rows, const float* w1, float* y1,
+                    const float* w2, float* y2, long ldy) {
+    const vox_hybrid_config& c = m->cfg;
+    if (c.norm_kind == VOX_NORM_RMS_GROUPS) {
+        hipLaunchKernelGGL(k_hb_rms_groups, dim3(n), dim3(256), 0, st, x, ldx, rows, w1, y1, w2, y2, ldy, c.width, c.norm_groups, c.eps);
+    } else {
+        hb_layernorm(st, n, x, ldx, rows, w1, y1, ldy, c.width, c.eps);
+        if (w2) hb_layernorm(st, n, x, ldx, rows, w2, y2, ldy, c.width, c.eps);
+    }
+}
+// the fused one-row norm + GEMV exists for the layer norm only
+template <typename T>
+static bool hb_try_norm_gemv(const vox_hybrid* m, hipStream_t st, int epi, const float* X, long ldx, const int* rows, const float* nw, const T* W,
+                             const float* bias, float* C, int N, int K) {
+    return m->cfg.norm_kind == VOX_NORM_LAYER && hb_try_ln_gemv<T>(st, epi, X, ldx, rows, nw, m->cfg.eps, W, bias, C, N, K);
+}
+
+// One mixer: reads the normed rows (hn != NULL) or norms `cur` itself with L.norm1, adds out_scale * mixer(.) to cur.
+template <typename T>
+static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const vox_hybrid_layer& L, void* cache, float* pool, float* state,
+                    const float* hn, float* cur, long ldx, int n, int n_req, int max_kvlen) {
+    const vox_hybrid_config& c = m->cfg;
+    const int W = c.width, ps = c.page_size;
+    const int n_in = hb_layer_in(L), n_proj = hb_layer_proj(L), n_mix = L.heads * L.vdim;
+    if (L.kind == VOX_MIXER_SHIFT_DECAY) {
+        // five token-shift mixes of the normed input, each with its own projection
+        if (!hn) { hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, nullptr, nullptr, (long)W); hn = m->h; }
+        const int HD = L.heads * L.dim;
+        const long per_slot = (long)HD * L.dim + W, rows_stride = (long)c.max_rows * W;
+        hipLaunchKernelGGL(k_hb_shift_mix, dim3(n), dim3(256), 0, st, hn, (long)W, L.shift_mu, m->shift, rows_stride, state, per_slot,
+                           (long)HD * L.dim, io->pos, io->row_req, io->req_rows, io->req_state, W);
+        const T* wi = (const T*)L.w_in;
+        for (int s2 = 0; s2 < 4; ++s2)
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->shift + s2 * rows_stride, W, wi + (size_t)s2 * HD * W, L.b_in ? L.b_in + s2 * HD : nullptr,
+                               m->proj + s2 * HD, n_proj, n, HD, W));
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_TANH, m->shift + 4 * rows_stride, W, wi + (size_t)4 * HD * W, nullptr, m->proj + 4 * HD, n_proj, n, L.lora, W));
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + 4 * HD, n_proj, (const T*)L.w_decay2, L.decay0, m->proj + 4 * HD + L.lora, n_proj, n, HD, L.lora));
+        const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
+        const int nwv = (L.dim + dpw - 1) / dpw, dpad = nwv * dpw;
+        const int tt = 4096 / dpad >= 16 ? 16 : (4096 / dpad >= 1 ? 4096 / dpad : 1);
+        auto kern = dpw == 16 ? k_hb_shift_decay_scan<16> : (dpw == 32 ? k_hb_shift_decay_scan<32> : k_hb_shift_decay_scan<64>);
+        const size_t lds = (size_t)(3 * tt * dpad + tt * 64 + 2 * nwv * 64) * 4;
+        hipLaunchKernelGGL(kern, dim3(n_req, L.heads, (L.dim + 63) / 64), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
+                           state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt);
+        hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj, 3 * HD,
+                           (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
+        return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
+    }
+    if (!hn && !(n == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, nullptr, L.norm1, (const T*)L.w_in, L.b_in, m->proj, n_in, W))) {
+        hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, nullptr, nullptr, (long)W);
+        hn = m->h;
+    }
+    if (hn) VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, hn, W, (const T*)L.w_in, L.b_in, m->proj, n_proj, n, n_in, W));
+    const int vt = (L.vdim + 63) / 64;
+    // dims per wave of the scans: the smallest of 16 / 32 / 64 that covers dim with at most 16 waves
+    const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
+    const int nwv = (L.dim + dpw - 1) / dpw;
+    // tokens staged per tile: as many as fit 4096 staged floats per array, at most 16
+    const int dpad = nwv * dpw;
+    const int tt = 4096 / dpad >= 16 ? 16 : (4096 / dpad >= 1 ? 4096 / dpad : 1);
+    if (L.kind == VOX_MIXER_HGRN2) {
+        auto kern = dpw == 16 ? k_hb_hgrn2_scan<16> : (dpw == 32 ? k_hb_hgrn2_scan<32> : k_hb_hgrn2_scan<64>);
+        const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + 2 * nwv * 64) * 4;
+        hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.lower,
+                           state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, tt);
+        hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 0, m->proj, (long)n_proj, -1,
+                           (int)HB_GATE_NONE, L.vdim, c.eps, L.out_scale);
+    } else if (L.kind == VOX_MIXER_MLSTM) {
+        auto kern = dpw == 16 ? k_hb_mlstm_scan<16> : (dpw == 32 ? k_hb_mlstm_scan<32> : k_hb_mlstm_scan<64>);
+        const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + tt * 2 + 2 * nwv * 65) * 4;
+        hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, state,
+                           io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap, tt);
+        hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj,
+                           2 * L.heads * L.dim + L.heads * L.vdim, (int)HB_GATE_SIGMOID, L.vdim, c.eps, L.out_scale);
+    } else if (L.kind == VOX_MIXER_RGLRU) {
+        const int C = L.heads * L.dim, bs = L.dim;
+        hipLaunchKernelGGL(k_hb_conv_causal, dim3(n, (C + 255) / 256), dim3(256), 0, st, m->proj, (long)n_proj, L.conv_w, L.conv_b, state, io->pos,
+                           io->row_req, io->req_rows, io->req_state, C, L.conv_taps);
+        // block-diagonal gates: block b's 2*bs outputs (r rows, then i rows) from its bs channels of the convolution's output
+        for (int b = 0; b < L.heads; ++b)
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + 2 * C + b * bs, n_proj, (const T*)L.w_gates + (size_t)b * 2 * bs * bs,
+                               L.b_gates ? L.b_gates + (size_t)b * 2 * bs : nullptr, m->proj + 3 * C + (size_t)b * 2 * bs, n_proj, n, 2 * bs, bs));
+        hipLaunchKernelGGL(k_hb_rglru_scan, dim3(n_req, (C + 63) / 64), dim3(64), 0, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.lam, state,
+                           io->req_rows, io->req_state, io->pos, C, bs, L.conv_taps, L.rec_scale, L.out_scale);
+    } else {
+        const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN;
+        const int H = L.heads, G = L.kv_heads, QG = H / G;
+        const int window = causal ? c.max_seq_len : L.window, P = causal ? 1 : L.pool;
+        const long v_base = (long)c.max_pages * ps * G * L.dim;
+        const int ppp = (ps - 1) / P + 1;
+        const bool one_row_each = n == n_req;      // decode steps: every block a row closes was filled by earlier steps
+        const hb_qkv_opts op = causal ? hb_qkv_opts{L.q_norm, L.k_norm, L.q_temp_coef, L.q_temp_every > 0 ? L.q_temp_every : 1, L.v_unit_rms}
+                                      : hb_qkv_opts{nullptr, nullptr, 0.f, 1, 0};
+        hipLaunchKernelGGL((k_hb_attn_prep<T>), dim3(n, H + G), dim3(64), 0, st, m->proj, (long)n_proj, (T*)cache, L.inv_freq, io->pos,
+                           io->page, io->slot, H, G, L.dim, L.vdim, causal ? 0 : L.rot_dims, ps, v_base, c.eps,
+                           one_row_each && !causal ? pool : (float*)nullptr, io->row_req, io->page_table, io->pt_stride, P, ppp, op);
+        if (!one_row_each && !causal)
+            hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)cache, pool, io->pos, io->row_req,
+                               io->page_table, io->pt_stride, G, L.dim, L.vdim, P, ps, ppp, v_base);
+        const int split = 16 / QG >= 4 ? 4 : (16 / QG >= 1 ? 16 / QG : 1);      // up to 16 waves per block, at most 4 per head
+        const int nwv2 = QG * split, dimp = (L.dim + 3) & ~3;
+        const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (L.vdim + 2) * 4;
+        // steps of few rows: 4-chunk key segments on separate blocks + a merge pass (more blocks than rows x kv heads); a row's
+        // result differs from the one-block form by the rounding of the merge only
+        const int max_keys = causal ? max_kvlen : (max_kvlen < window ? max_kvlen : window) + max_kvlen / P + 1;
+        const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
+        const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (L.vdim + 2) * 4 <= m->attn_ws_bytes;
+        hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, m->proj, (long)n_proj, (const T*)cache,
+                           pool, m->mix, (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, window,
+                           P, ps, ppp, v_base, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr,
+                           causal ? 0 : 1, L.out_scale);
+        if (segmented)
+            hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->proj, (long)n_proj, m->mix, (long)n_mix,
+                               io->pos, H, G, L.dim, L.vdim, window, P, HB_ATTN_SEG, causal ? 0 : 1, L.out_scale);
+    }
+    return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
+}
+
+// Routed feed-forward of the normed rows h2, added to cur.  Few rows: one GEMV pair per routed entry; more: the entries are
+// listed per expert and every expert multiplies its own rows in one tile launch.
+#define HB_MOE_GEMV_ROWS 8
+template <typename T>
+static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const float* h2, float* cur, long ldx, int n) {
+    const int W = m->cfg.width, nE = E.experts + E.identity, top = E.top, ne = n * top, ff = E.ff;
+    VOX_TRY(hb_gemm<float>(st, HB_EPI_STORE, h2, W, E.router, nullptr, m->moe_z, nE, n, nE, W));
+    hipLaunchKernelGGL(k_hb_moe_route, dim3(n), dim3(64), (size_t)(2 * nE + top) * 4, st, m->moe_z, E.correction, nE, top, m->moe_sel, m->moe_wgt);
+    if (E.experts > 0) {
+        if (n <= HB_MOE_GEMV_ROWS) {
+            hipLaunchKernelGGL((k_hb_moe_gemv<T, true>), dim3((ff + 3) / 4, ne), dim3(256), 0, st, h2, (long)W, top, (const T*)E.w_gate_up,
+                               (long)2 * ff * W, m->moe_sel, E.experts, m->moe_act, (long)ff, ff, W, E.limit, E.act_alpha);
+            hipLaunchKernelGGL((k_hb_moe_gemv<T, false>), dim3((W + 3) / 4, ne), dim3(256), 0, st, m->moe_act, (long)ff, 1, (const T*)E.w_down,
+                               (long)W * ff, m->moe_sel, E.experts, m->moe_out, (long)W, W, ff, 0.f, 0.f);
+        } else {
+            const int cap = m->cfg.max_rows;
+            hipLaunchKernelGGL(k_hb_moe_group, dim3(E.experts), dim3(256), 0, st, m->moe_sel, ne, cap, m->moe_list, m->moe_count);
+            VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, h2, (long)W, (const T*)E.w_gate_up, nullptr, m->ff, (long)2 * ff, n, 2 * ff, W,
+                                                hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)2 * ff * W}, E.experts));
+            hipLaunchKernelGGL(k_hb_glu_clamp, dim3(ne, (ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, ff, E.limit, E.act_alpha,
+                               m->moe_sel, E.experts);
+            VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, m->moe_act, (long)ff, (const T*)E.w_down, nullptr, m->moe_out, (long)W, n, W, ff,
+                                                hb_rowmap{m->moe_count, m->moe_list, cap, 1, (long)W * ff}, E.experts));
+        }
+    }
+    hipLaunchKernelGGL(k_hb_moe_combine, dim3(n), dim3(256), 0, st, cur, ldx, h2, (long)W, m->moe_out, m->moe_sel, m->moe_wgt, top, E.experts, W);
+    if (E.shared_ff > 0) {
+        const int sf = E.shared_ff;
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, h2, W, (const T*)E.shared_gate_up, nullptr, m->ff, 2 * sf, n, 2 * sf, W));
+        hipLaunchKernelGGL(k_hb_glu_clamp, dim3(n, (sf + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, sf, E.shared_limit, E.act_alpha,
+                           (const int*)nullptr, 0);
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->moe_act, sf, (const T*)E.shared_down, nullptr, cur, ldx, n, W, sf));
+    }
+    return VOX_OK;
 }
 
 template <typename T>
 static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const int32_t* ids, int n, int n_req, int n_out, int max_kvlen) {
     const vox_hybrid_config& c = m->cfg;
-    const int W = c.width, ps = c.page_size;
+    const int W = c.width;
     const long ldx = 2L * W;
-    hipLaunchKernelGGL((k_hb_embed<T>), dim3(n), dim3(256), 0, st, (const T*)m->w.embedding, ids, 1, m->xa, m->xb, W, c.vocab);
+    hipLaunchKernelGGL((k_hb_embed<T>), dim3(n), dim3(256), 0, st, (const T*)m->w.embedding, ids, 1, m->xa, m->xb, W, c.vocab, c.embed_scale);
     float *cur = m->xa, *other = m->xb;
     for (int ri = 0; ri < c.n_runs; ++ri) {
         const vox_hybrid_run& run = m->runs[ri];
@@ -1215,62 +1793,25 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, cur, ldx, (const T*)m->w.loop_in, nullptr, other, ldx, n, W, 2 * W));
             float* t = cur; cur = other; other = t;
         }
-        const int n_in = hb_layer_in(L), n_mix = L.heads * L.vdim;
-        if (!(n == 1 && hb_try_ln_gemv<T>(st, HB_EPI_STORE, cur, ldx, nullptr, L.norm1, c.eps, (const T*)L.w_in, L.b_in, m->proj, n_in, W))) {
-            hb_layernorm(st, n, cur, ldx, nullptr, L.norm1, m->h, (long)W, W, c.eps);
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->h, W, (const T*)L.w_in, L.b_in, m->proj, n_in, n, n_in, W));
+        const bool has_ff = L.ff > 0 || L.moe;
+        const bool parallel = L.block == VOX_BLOCK_PARALLEL;
+        // a parallel layer norms x once for both branches before anything is added; a mixer with a sibling needs the normed rows twice
+        const float* hn = nullptr;
+        if (parallel || L.sibling >= 0) {
+            hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, parallel && has_ff ? L.norm2 : nullptr, m->h2, (long)W);
+            hn = m->h;
         }
-        const int vt = (L.vdim + 63) / 64;
-        // dims per wave of the scans: the smallest of 16 / 32 / 64 that covers dim with at most 16 waves
-        const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
-        const int nwv = (L.dim + dpw - 1) / dpw;
-        // tokens staged per tile: as many as fit 4096 staged floats per array, at most 16
-        const int dpad = nwv * dpw;
-        const int tt = 4096 / dpad >= 16 ? 16 : (4096 / dpad >= 1 ? 4096 / dpad : 1);
-        if (L.kind == VOX_MIXER_HGRN2) {
-            auto kern = dpw == 16 ? k_hb_hgrn2_scan<16> : (dpw == 32 ? k_hb_hgrn2_scan<32> : k_hb_hgrn2_scan<64>);
-            const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + 2 * nwv * 64) * 4;
-            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, L.lower,
-                               run.state, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, tt);
-            hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 0, m->proj, (long)n_in, -1,
-                               L.vdim, c.eps);
-        } else if (L.kind == VOX_MIXER_MLSTM) {
-            auto kern = dpw == 16 ? k_hb_mlstm_scan<16> : (dpw == 32 ? k_hb_mlstm_scan<32> : k_hb_mlstm_scan<64>);
-            const size_t lds = (size_t)(2 * tt * dpad + tt * 64 + tt * 2 + 2 * nwv * 65) * 4;
-            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_in, m->mix, (long)n_mix, run.state,
-                               io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.vdim, L.gate_cap, tt);
-            hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_in,
-                               2 * L.heads * L.dim + L.heads * L.vdim, L.vdim, c.eps);
-        } else {
-            const int H = L.heads, G = L.kv_heads, QG = H / G;
-            const long v_base = (long)c.max_pages * ps * G * L.dim;
-            const int ppp = (ps - 1) / L.pool + 1;
-            const bool one_row_each = n == n_req;      // decode steps: every block a row closes was filled by earlier steps
-            hipLaunchKernelGGL((k_hb_attn_prep<T>), dim3(n, H + G), dim3(64), 0, st, m->proj, (long)n_in, (T*)run.cache, L.inv_freq, io->pos,
-                               io->page, io->slot, H, G, L.dim, L.vdim, L.rot_dims, ps, v_base, c.eps, one_row_each ? run.pool : (float*)nullptr,
-                               io->row_req, io->page_table, io->pt_stride, L.pool, ppp);
-            if (!one_row_each)
-                hipLaunchKernelGGL((k_hb_pool_update<T>), dim3(n, G), dim3(64), 0, st, (const T*)run.cache, run.pool, io->pos, io->row_req,
-                                   io->page_table, io->pt_stride, G, L.dim, L.vdim, L.pool, ps, ppp, v_base);
-            const int split = 16 / QG >= 4 ? 4 : (16 / QG >= 1 ? 16 / QG : 1);      // up to 16 waves per block, at most 4 per head
-            const int nwv2 = QG * split, dimp = (L.dim + 3) & ~3;
-            const size_t lds = (size_t)nwv2 * 64 * 8 + (size_t)nwv2 * 64 * 4 + (size_t)QG * dimp * 4 + (size_t)nwv2 * (L.vdim + 2) * 4;
-            // steps of few rows: 4-chunk key segments on separate blocks + a merge pass (more blocks than rows x kv heads); a row's
-            // result differs from the one-block form by the rounding of the merge only
-            const int max_keys = (max_kvlen < L.window ? max_kvlen : L.window) + max_kvlen / L.pool + 1;
-            const int nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
-            const bool segmented = n <= HB_ATTN_SEG_ROWS && nseg > 1 && (size_t)n * H * nseg * (L.vdim + 2) * 4 <= m->attn_ws_bytes;
-            hipLaunchKernelGGL((k_hb_attn<T>), dim3(n, G, segmented ? nseg : 1), dim3(64 * nwv2), lds, st, m->proj, (long)n_in, (const T*)run.cache,
-                               run.pool, m->mix, (long)n_mix, io->pos, io->row_req, io->page_table, io->pt_stride, H, G, L.dim, L.vdim, L.window,
-                               L.pool, ps, ppp, v_base, L.scale, split, segmented ? HB_ATTN_SEG : 0, segmented ? m->attn_ws : (float*)nullptr);
-            if (segmented)
-                hipLaunchKernelGGL(k_hb_attn_merge, dim3(n, H), dim3(64), 0, st, m->attn_ws, nseg, m->proj, (long)n_in, m->mix, (long)n_mix,
-                                   io->pos, H, G, L.dim, L.vdim, L.window, L.pool, HB_ATTN_SEG);
-        }
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix));
-        if (L.ff > 0) {
-            if (!(n == 1 && hb_try_ln_gemv<T>(st, HB_EPI_GELU, cur, ldx, nullptr, L.norm2, c.eps, (const T*)L.w_up, nullptr, m->ff, L.ff, W))) {
-                hb_layernorm(st, n, cur, ldx, nullptr, L.norm2, m->h, (long)W, W, c.eps);
+        VOX_TRY(hb_mixer<T>(m, st, io, L, run.cache, run.pool, run.state, hn, cur, ldx, n, n_req, max_kvlen));
+        if (L.sibling >= 0)
+            VOX_TRY(hb_mixer<T>(m, st, io, m->layers[L.sibling], run.side_cache, run.side_pool, run.side_state, hn, cur, ldx, n, n_req, max_kvlen));
+        if (L.moe) {
+            if (!parallel) hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h2, nullptr, nullptr, (long)W);
+            VOX_TRY(hb_moe<T>(m, st, *L.moe, m->h2, cur, ldx, n));
+        } else if (L.ff > 0) {
+            if (parallel) {
+                VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h2, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
+            } else if (!(n == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_GELU, cur, ldx, nullptr, L.norm2, (const T*)L.w_up, nullptr, m->ff, L.ff, W))) {
+                hb_norm(m, st, n, cur, ldx, nullptr, L.norm2, m->h, nullptr, nullptr, (long)W);
                 VOX_TRY(hb_gemm<T>(st, HB_EPI_GELU, m->h, W, (const T*)L.w_up, nullptr, m->ff, L.ff, n, L.ff, W));
             }
             VOX_TRY(hb_gemm<T>(st, HB_EPI_RESID, m->ff, L.ff, (const T*)L.w_down, nullptr, cur, ldx, n, W, L.ff));
@@ -1279,9 +1820,9 @@ static int hb_step(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, const
             hipLaunchKernelGGL(k_hb_copy_rows, dim3(n), dim3(256), 0, st, cur, ldx, io->trace + (size_t)ri * c.max_rows * W, (long)W, W);
     }
     if (n_out > 0) {
-        if (!(n_out == 1 && hb_try_ln_gemv<T>(st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, c.eps, (const T*)m->w.head, nullptr,
-                                              io->logits, c.vocab, W))) {
-            hb_layernorm(st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, (long)W, W, c.eps);
+        if (!(n_out == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, io->out_rows, m->w.final_norm, (const T*)m->w.head, nullptr,
+                                                io->logits, c.vocab, W))) {
+            hb_norm(m, st, n_out, cur, ldx, io->out_rows, m->w.final_norm, m->hout, nullptr, nullptr, (long)W);
             VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->hout, W, (const T*)m->w.head, nullptr, io->logits, c.vocab, n_out, c.vocab, W));
         }
     }
@@ -1296,51 +1837,101 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
     if (cfg->dtype != VOX_HYBRID_BF16 && cfg->dtype != VOX_HYBRID_F32) return vox_fail(VOX_ERR_INVALID, "hybrid_create: dtype %d", cfg->dtype);
     if (cfg->width < 1 || cfg->vocab < 1 || cfg->page_size < 1 || cfg->max_rows < 1 || cfg->max_batch < 1 || cfg->max_out < 1 || cfg->max_seq_len < 1)
         return vox_fail(VOX_ERR_INVALID, "hybrid_create: bad sizes");
+    if (cfg->norm_kind != VOX_NORM_LAYER && cfg->norm_kind != VOX_NORM_RMS_GROUPS) return vox_fail(VOX_ERR_INVALID, "hybrid_create: norm kind %d", cfg->norm_kind);
+    if (cfg->norm_kind == VOX_NORM_RMS_GROUPS && (cfg->norm_groups < 1 || cfg->width % cfg->norm_groups != 0))
+        return vox_fail(VOX_ERR_INVALID, "hybrid_create: %d norm groups do not divide width %d", cfg->norm_groups, cfg->width);
     vox_hybrid* m = new vox_hybrid();
     m->ctx = ctx; m->cfg = *cfg; m->w = *w;
     m->layers.assign(w->layers, w->layers + cfg->n_layers);
     m->runs.assign(w->runs, w->runs + cfg->n_runs);
     m->w.layers = nullptr; m->w.runs = nullptr;
+    m->moes.reserve(m->layers.size());
+    for (vox_hybrid_layer& L : m->layers)
+        if (L.moe) { m->moes.push_back(*L.moe); L.moe = &m->moes.back(); }
     for (const vox_hybrid_layer& L : m->layers) {
         const int n_in = hb_layer_in(L);
         const char* bad = nullptr;
         if (n_in < 0) bad = "unknown mixer kind";
         else if (L.heads < 1 || L.dim < 1 || L.vdim < 1) bad = "heads / dim / vdim";
-        else if (L.vdim > 64 * HB_MAX_VPL) bad = "vdim above 512";
+        else if (L.vdim > 64 * HB_MAX_VPL && L.kind != VOX_MIXER_RGLRU) bad = "vdim above 512";
         else if (!L.norm1 || !L.w_in || !L.w_out) bad = "missing weights";
         else if (L.ff > 0 && (!L.norm2 || !L.w_up || !L.w_down)) bad = "missing feed-forward weights";
+        else if (L.block != VOX_BLOCK_SEQUENTIAL && L.block != VOX_BLOCK_PARALLEL) bad = "block form";
+        else if (L.sibling >= cfg->n_layers || (L.sibling >= 0 && m->layers[L.sibling].sibling >= 0)) bad = "sibling index";
         else if (L.kind == VOX_MIXER_HGRN2 && (!L.lower || !L.head_norm)) bad = "hgrn2 needs lower and head_norm";
         else if (L.kind == VOX_MIXER_MLSTM && (!L.head_norm || !(L.gate_cap > 0.f))) bad = "mlstm needs head_norm and gate_cap";
-        else if (L.kind != VOX_MIXER_POOLED_WINDOW_ATTN && L.dim > 64 * HB_SCAN_MAX_WAVES) bad = "recurrent dim above 1024";
-        else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN) {
+        else if ((L.kind == VOX_MIXER_HGRN2 || L.kind == VOX_MIXER_MLSTM || L.kind == VOX_MIXER_SHIFT_DECAY) && L.dim > 64 * HB_SCAN_MAX_WAVES)
+            bad = "recurrent dim above 1024";
+        else if (L.kind == VOX_MIXER_RGLRU && (L.dim != L.vdim || L.conv_taps < 1 || !L.conv_w || !L.w_gates || !L.lam)) bad = "rglru needs conv, gates and lam";
+        else if (L.kind == VOX_MIXER_SHIFT_DECAY && (L.dim != L.vdim || L.lora < 1 || !L.shift_mu || !L.w_decay2 || !L.decay0 || !L.bonus || !L.head_norm))
+            bad = "shift-decay needs mu, decay and bonus tensors";
+        else if (hb_is_attn(L.kind)) {
             if (L.kv_heads < 1 || L.heads % L.kv_heads != 0 || L.heads / L.kv_heads > 16) bad = "heads / kv_heads (group of at most 16)";
             else if (L.dim > 64 * HB_MAX_DPL) bad = "dim above 512";
-            else if (L.window < 1 || L.pool < 1) bad = "window / pool";
-            else if (L.rot_dims < 0 || L.rot_dims > L.dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq)) bad = "rot_dims";
+            else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && (L.window < 1 || L.pool < 1)) bad = "window / pool";
+            else if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && (L.rot_dims < 0 || L.rot_dims > L.dim || (L.rot_dims & 1) || (L.rot_dims > 0 && !L.inv_freq))) bad = "rot_dims";
+        }
+        if (!bad && L.moe) {
+            const vox_hybrid_moe& E = *L.moe;
+            if (E.experts < 0 || E.identity < 0 || E.top < 1 || E.top > E.experts + E.identity) bad = "moe: experts / identity / top";
+            else if (!E.router || !L.norm2) bad = "moe: router or norm2 missing";
+            else if (E.experts > 0 && (E.ff < 1 || !E.w_gate_up || !E.w_down)) bad = "moe: expert weights";
+            else if (E.shared_ff > 0 && (!E.shared_gate_up || !E.shared_down)) bad = "moe: shared expert weights";
         }
         if (bad) { delete m; return vox_fail(VOX_ERR_INVALID, "hybrid_create: layer: %s", bad); }
-        if (n_in > m->max_in) m->max_in = n_in;
+        const int n_proj = hb_layer_proj(L);
+        if (n_proj > m->max_in) m->max_in = n_proj;
         if (L.heads * L.vdim > m->max_mix) m->max_mix = L.heads * L.vdim;
         if (L.ff > m->max_ff) m->max_ff = L.ff;
+        if (L.kind == VOX_MIXER_SHIFT_DECAY) m->any_shift = true;
+        if (L.moe) {
+            const vox_hybrid_moe& E = *L.moe;
+            if (E.experts + E.identity > m->max_ne) m->max_ne = E.experts + E.identity;
+            if (E.experts > m->max_experts) m->max_experts = E.experts;
+            if (E.top > m->max_top) m->max_top = E.top;
+            if (E.top * 2 * E.ff > m->max_ff) m->max_ff = E.top * 2 * E.ff;
+            if (2 * E.shared_ff > m->max_ff) m->max_ff = 2 * E.shared_ff;
+            if (E.top * E.ff > m->max_eff) m->max_eff = E.top * E.ff;
+            if (E.shared_ff > m->max_eff) m->max_eff = E.shared_ff;
+        }
     }
     for (const vox_hybrid_run& r : m->runs) {
         const char* bad = nullptr;
         if (r.layer < 0 || r.layer >= cfg->n_layers) bad = "layer index";
-        else if (m->layers[r.layer].kind == VOX_MIXER_POOLED_WINDOW_ATTN ? (!r.cache || !r.pool) : !r.state) bad = "missing cache / state";
-        else if (r.loop_in && !w->loop_in) bad = "loop_in weight";
+        else {
+            const vox_hybrid_layer& L = m->layers[r.layer];
+            if (hb_is_attn(L.kind) ? (!r.cache || (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN && !r.pool)) : !r.state) bad = "missing cache / state";
+            else if (L.sibling >= 0) {
+                const vox_hybrid_layer& S2 = m->layers[L.sibling];
+                if (hb_is_attn(S2.kind) ? (!r.side_cache || (S2.kind == VOX_MIXER_POOLED_WINDOW_ATTN && !r.side_pool)) : !r.side_state)
+                    bad = "missing cache / state of the sibling mixer";
+            }
+            if (!bad && r.loop_in && !w->loop_in) bad = "loop_in weight";
+        }
         if (bad) { delete m; return vox_fail(VOX_ERR_INVALID, "hybrid_create: run: %s", bad); }
     }
     const size_t R = cfg->max_rows, W = cfg->width;
     bool ok = hipMalloc((void**)&m->xa, R * 2 * W * 4) == hipSuccess && hipMalloc((void**)&m->xb, R * 2 * W * 4) == hipSuccess &&
-              hipMalloc((void**)&m->h, R * W * 4) == hipSuccess && hipMalloc((void**)&m->proj, R * (size_t)m->max_in * 4) == hipSuccess &&
+              hipMalloc((void**)&m->h, R * W * 4) == hipSuccess && hipMalloc((void**)&m->h2, R * W * 4) == hipSuccess &&
+              hipMalloc((void**)&m->proj, R * (size_t)m->max_in * 4) == hipSuccess &&
               hipMalloc((void**)&m->mix, R * (size_t)m->max_mix * 4) == hipSuccess &&
               hipMalloc((void**)&m->ff, R * (size_t)(m->max_ff > 0 ? m->max_ff : 1) * 4) == hipSuccess &&
               hipMalloc((void**)&m->hout, (size_t)cfg->max_out * W * 4) == hipSuccess &&
               hipMalloc((void**)&m->logits16, (size_t)cfg->max_batch * cfg->vocab * 2) == hipSuccess;
+    if (ok && m->any_shift) ok = hipMalloc((void**)&m->shift, 5 * R * W * 4) == hipSuccess;
+    if (ok && m->max_top > 0) {
+        const size_t ne = R * (size_t)m->max_top;
+        ok = hipMalloc((void**)&m->moe_z, R * (size_t)m->max_ne * 4) == hipSuccess && hipMalloc((void**)&m->moe_wgt, ne * 4) == hipSuccess &&
+             hipMalloc((void**)&m->moe_sel, ne * 4) == hipSuccess && hipMalloc((void**)&m->moe_act, R * (size_t)(m->max_eff > 0 ? m->max_eff : 1) * 4) == hipSuccess &&
+             hipMalloc((void**)&m->moe_out, ne * W * 4) == hipSuccess &&
+             hipMalloc((void**)&m->moe_list, (size_t)(m->max_experts > 0 ? m->max_experts : 1) * R * 4) == hipSuccess &&
+             hipMalloc((void**)&m->moe_count, (size_t)(m->max_experts > 0 ? m->max_experts : 1) * 4) == hipSuccess;
+    }
     // partial results of segmented attention launches: few rows x heads x segments of the longest sequence
     for (const vox_hybrid_layer& L : m->layers)
-        if (L.kind == VOX_MIXER_POOLED_WINDOW_ATTN) {
-            const int max_keys = (cfg->max_seq_len < L.window ? cfg->max_seq_len : L.window) + cfg->max_seq_len / L.pool + 1;
+        if (hb_is_attn(L.kind)) {
+            const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN;
+            const int max_keys = causal ? cfg->max_seq_len : (cfg->max_seq_len < L.window ? cfg->max_seq_len : L.window) + cfg->max_seq_len / L.pool + 1;
             const size_t nseg = ((max_keys + 63) / 64 + HB_ATTN_SEG - 1) / HB_ATTN_SEG;
             const size_t b = (size_t)HB_ATTN_SEG_ROWS * L.heads * nseg * (L.vdim + 2) * 4;
             if (b > m->attn_ws_bytes) m->attn_ws_bytes = b;
@@ -1353,8 +1944,10 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
 
 void vox_hybrid_destroy(vox_hybrid* m) {
     if (!m) return;
-    (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->proj); (void)hipFree(m->mix);
-    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws);
+    (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->h2); (void)hipFree(m->proj); (void)hipFree(m->mix);
+    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws); (void)hipFree(m->shift);
+    (void)hipFree(m->moe_z); (void)hipFree(m->moe_wgt); (void)hipFree(m->moe_sel); (void)hipFree(m->moe_act); (void)hipFree(m->moe_out);
+    (void)hipFree(m->moe_list); (void)hipFree(m->moe_count);
     delete m;
 }
 

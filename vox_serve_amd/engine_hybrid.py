@@ -1,5 +1,7 @@
-"""Host side of `vox_hybrid_*`: the engine for decoders that mix tokens with linear recurrences (HGRN2, mLSTM) and with
-sliding-window attention over a paged cache with pooled history, optionally looping a range of layers over shared weights.
+"""Host side of `vox_hybrid_*`: the engine for decoders that mix tokens with linear recurrences (HGRN2, mLSTM, a real-gated
+diagonal unit behind a short convolution, a matrix state with token shift and per-channel decay) and with attention over a paged
+cache (a sliding window with pooled history, or plain causal attention with normed q / k / v), optionally two mixers side by
+side, sequential or parallel layers, a dense or a routed feed-forward, and a range of layers looped over shared weights.
 
 It reuses the plan / stream / hipGraph machinery of the other LM engines (`Qwen3Engine`): one pinned int32 plan block per
 step, decode steps captured per batch size.  Beyond the K / V pages that the worker hands out, every request holds one
@@ -17,16 +19,33 @@ import torch
 from . import _native as N
 from .engine import Qwen3Engine
 
-MIXER_HGRN2, MIXER_POOLED_WINDOW_ATTN, MIXER_MLSTM = 0, 1, 2
-MIXER_KINDS = {"hgrn2": MIXER_HGRN2, "attention": MIXER_POOLED_WINDOW_ATTN, "mlstm": MIXER_MLSTM}
+MIXER_HGRN2, MIXER_POOLED_WINDOW_ATTN, MIXER_MLSTM, MIXER_RGLRU, MIXER_CAUSAL_ATTN, MIXER_SHIFT_DECAY = 0, 1, 2, 3, 4, 5
+MIXER_KINDS = {"hgrn2": MIXER_HGRN2, "attention": MIXER_POOLED_WINDOW_ATTN, "mlstm": MIXER_MLSTM, "rglru": MIXER_RGLRU,
+               "causal_attention": MIXER_CAUSAL_ATTN, "shift_decay": MIXER_SHIFT_DECAY}
+ATTENTION_KINDS = ("attention", "causal_attention")
+NORM_KINDS = {"layer": 0, "rms_groups": 1}
+BLOCK_FORMS = {"sequential": 0, "parallel": 1}
+
+
+@dataclass
+class MoECfg:
+    """Routed feed-forward: `experts` clamped gated units + `identity` pass-through outputs, `top` per token, optional shared expert."""
+    experts: int
+    identity: int
+    top: int
+    ff: int
+    limit: float
+    shared_ff: int = 0
+    shared_limit: float = 0.0
+    act_alpha: float = 1.702
 
 
 @dataclass
 class MixerCfg:
-    kind: str                       # "hgrn2" | "attention" | "mlstm"
-    heads: int
-    dim: int
-    vdim: int
+    kind: str                       # a key of MIXER_KINDS
+    heads: int                      # rglru: blocks of the gate matrices
+    dim: int                        # rglru: channels per block
+    vdim: int                       # rglru, shift_decay: = dim
     kv_heads: int = 0               # attention
     window: int = 0                 # attention: tokens a position sees, itself included
     pool: int = 0                   # attention: tokens per pooled block
@@ -35,7 +54,17 @@ class MixerCfg:
     rot_factor: float = 1.0         # linear position scaling: every rotary frequency is divided by it
     scale: float = 1.0              # attention score scale
     gate_cap: float = 0.0           # mLSTM: soft cap of the gate pre-activations
-    ff: int = 0                     # feed-forward width (0: none)
+    ff: int = 0                     # dense feed-forward width (0: none)
+    q_temp_coef: float = 0.0        # causal attention: q *= 1 + coef * ln(floor((p + 1) / every) + 1)
+    q_temp_every: int = 1
+    v_unit_rms: bool = False        # causal attention: values divided by their RMS per head before they are cached
+    conv_taps: int = 0              # rglru: taps of the causal convolution
+    rec_scale: float = 8.0          # rglru: a = exp(-rec_scale * r * softplus(lam))
+    lora: int = 0                   # shift_decay: width of the decay bottleneck
+    out_scale: float = 1.0          # the mixer's output is multiplied by this before it joins the residual sum
+    block: str = "sequential"       # "sequential": x += mixer(norm1 x); x += ff(norm2 x) | "parallel": x += mixer(norm1 x) + ff(norm2 x)
+    side: Optional["MixerCfg"] = None   # a second mixer on the same normed input, added to the same sum
+    moe: Optional[MoECfg] = None    # routed feed-forward (instead of the dense one)
 
     @property
     def n_in(self) -> int:
@@ -45,7 +74,19 @@ class MixerCfg:
             return 2 * h * d + h * v
         if self.kind == "attention":
             return h * d + self.kv_heads * (d + v) + h
+        if self.kind == "rglru":
+            return 2 * h * d
+        if self.kind == "causal_attention":
+            return h * d + self.kv_heads * (d + v)
+        if self.kind == "shift_decay":
+            return 4 * h * d + self.lora
         return 2 * h * d + 2 * h * v + 2 * h
+
+    def state_floats(self, width: int) -> int:
+        """fp32 values of one recurrent-state slot (0 for attention)."""
+        h, d, v = self.heads, self.dim, self.vdim
+        return {"hgrn2": h * d * v, "mlstm": h * (d * v + d + 1), "rglru": max(self.conv_taps, 1) * h * d,
+                "shift_decay": h * d * d + width}.get(self.kind, 0)
 
 
 @dataclass
@@ -55,6 +96,9 @@ class HybridCfg:
     eps: float
     layers: List[MixerCfg] = field(default_factory=list)
     loop: Optional[tuple] = None    # (start, stop, times): layers start..stop-1 run `times` times in a row
+    norm_kind: str = "layer"        # "layer": weight-only layer norm | "rms_groups": RMS norm over norm_groups equal slices
+    norm_groups: int = 1
+    embed_scale: float = 1.0
 
     def runs(self):
         """[(layer index, loop_in)] in execution order; loop_in marks the first layer of every pass of the looped range."""
@@ -68,21 +112,36 @@ class HybridCfg:
         return out + [(i, False) for i in range(b, n)]
 
 
+class HybridMoEC(ctypes.Structure):
+    _fields_ = [(n, ctypes.c_int32) for n in ("experts", "identity", "top", "ff", "shared_ff")] + \
+               [(n, ctypes.c_float) for n in ("limit", "shared_limit", "act_alpha")] + \
+               [(n, ctypes.c_void_p) for n in ("router", "correction", "w_gate_up", "w_down", "shared_gate_up", "shared_down")]
+
+
 class HybridLayerC(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("kind", "heads", "kv_heads", "dim", "vdim", "window", "pool", "rot_dims")] + \
                [("scale", ctypes.c_float), ("gate_cap", ctypes.c_float), ("ff", ctypes.c_int32)] + \
                [(n, ctypes.c_void_p) for n in ("norm1", "norm2", "w_in", "b_in", "w_out", "lower", "head_norm", "inv_freq",
-                                               "w_up", "w_down")]
+                                               "w_up", "w_down")] + \
+               [("block", ctypes.c_int32), ("sibling", ctypes.c_int32), ("out_scale", ctypes.c_float),
+                ("q_norm", ctypes.c_void_p), ("k_norm", ctypes.c_void_p), ("q_temp_coef", ctypes.c_float),
+                ("q_temp_every", ctypes.c_int32), ("v_unit_rms", ctypes.c_int32),
+                ("conv_taps", ctypes.c_int32), ("rec_scale", ctypes.c_float), ("conv_w", ctypes.c_void_p), ("conv_b", ctypes.c_void_p),
+                ("w_gates", ctypes.c_void_p), ("b_gates", ctypes.c_void_p), ("lam", ctypes.c_void_p),
+                ("lora", ctypes.c_int32), ("shift_mu", ctypes.c_void_p), ("w_decay2", ctypes.c_void_p), ("decay0", ctypes.c_void_p),
+                ("bonus", ctypes.c_void_p), ("moe", ctypes.POINTER(HybridMoEC))]
 
 
 class HybridRunC(ctypes.Structure):
     _fields_ = [("layer", ctypes.c_int32), ("loop_in", ctypes.c_int32), ("cache", ctypes.c_void_p), ("pool", ctypes.c_void_p),
-                ("state", ctypes.c_void_p)]
+                ("state", ctypes.c_void_p), ("side_cache", ctypes.c_void_p), ("side_pool", ctypes.c_void_p),
+                ("side_state", ctypes.c_void_p)]
 
 
 class HybridConfigC(ctypes.Structure):
     _fields_ = [(n, ctypes.c_int32) for n in ("width", "vocab", "n_layers", "n_runs", "dtype", "page_size", "max_rows",
-                                              "max_batch", "max_out", "max_pages", "max_seq_len")] + [("eps", ctypes.c_float)]
+                                              "max_batch", "max_out", "max_pages", "max_seq_len")] + [("eps", ctypes.c_float)] + \
+               [("norm_kind", ctypes.c_int32), ("norm_groups", ctypes.c_int32), ("embed_scale", ctypes.c_float)]
 
 
 class HybridWeightsC(ctypes.Structure):
@@ -104,8 +163,10 @@ def rotary_frequencies(rot_dims: int, base: float, factor: float) -> torch.Tenso
 
 class HybridEngine(Qwen3Engine):
     """`weights`: {"embedding", "head", "final_norm", "loop_in" (or None), "layers": [per layer dict with norm1, norm2, w_in,
-    b_in, w_out, lower, head_norm, w_up, w_down]} — matrices in any float dtype (stored as the engine's dtype), vectors
-    stored as fp32.  dtype: torch.bfloat16 or torch.float32."""
+    b_in, w_out, lower, head_norm, w_up, w_down; per mixer kind also q_norm, k_norm | conv_w, conv_b, w_gates, b_gates, lam |
+    shift_mu, w_decay2, decay0, bonus; "moe": {router, correction, w_gate_up, w_down, shared_gate_up, shared_down}; "side":
+    the same mixer keys for a sibling mixer]} — matrices in any float dtype (stored as the engine's dtype), vectors and
+    the router stored as fp32.  dtype: torch.bfloat16 or torch.float32."""
 
     needs_state_slots = True
 
@@ -139,11 +200,13 @@ class HybridEngine(Qwen3Engine):
             return self._keep[-1].data_ptr()
 
         W = cfg.width
-        larr = (HybridLayerC * len(cfg.layers))()
-        for i, (m, lw) in enumerate(zip(cfg.layers, weights["layers"])):
-            assert tuple(lw["w_in"].shape) == (m.n_in, W), (i, tuple(lw["w_in"].shape), m.n_in)
-            assert tuple(lw["w_out"].shape) == (W, m.heads * m.vdim), (i, tuple(lw["w_out"].shape))
-            c = larr[i]
+        sides = [(i, m.side) for i, m in enumerate(cfg.layers) if m.side is not None]
+        larr = (HybridLayerC * (len(cfg.layers) + len(sides)))()
+        self._moes = []
+
+        def fill(c, m, lw, i):
+            assert tuple(lw["w_in"].shape) == (m.n_in, W), (i, m.kind, tuple(lw["w_in"].shape), m.n_in)
+            assert tuple(lw["w_out"].shape) == (W, m.heads * m.vdim), (i, m.kind, tuple(lw["w_out"].shape))
             c.kind, c.heads, c.kv_heads, c.dim, c.vdim = MIXER_KINDS[m.kind], m.heads, m.kv_heads, m.dim, m.vdim
             c.window, c.pool, c.rot_dims, c.scale, c.gate_cap, c.ff = m.window, m.pool, m.rot_dims, m.scale, m.gate_cap, m.ff
             c.norm1, c.norm2 = vec(lw["norm1"]), vec(lw.get("norm2"))
@@ -151,25 +214,56 @@ class HybridEngine(Qwen3Engine):
             c.lower, c.head_norm = vec(lw.get("lower")), vec(lw.get("head_norm"))
             c.inv_freq = vec(rotary_frequencies(m.rot_dims, m.rot_base, m.rot_factor)) if m.kind == "attention" and m.rot_dims else None
             c.w_up, c.w_down = mat(lw.get("w_up")), mat(lw.get("w_down"))
+            c.block, c.sibling, c.out_scale = BLOCK_FORMS[m.block], -1, m.out_scale
+            c.q_norm, c.k_norm = vec(lw.get("q_norm")), vec(lw.get("k_norm"))
+            c.q_temp_coef, c.q_temp_every, c.v_unit_rms = m.q_temp_coef, m.q_temp_every, int(m.v_unit_rms)
+            c.conv_taps, c.rec_scale = m.conv_taps, m.rec_scale
+            c.conv_w, c.conv_b, c.w_gates, c.b_gates, c.lam = vec(lw.get("conv_w")), vec(lw.get("conv_b")), mat(lw.get("w_gates")), \
+                vec(lw.get("b_gates")), vec(lw.get("lam"))
+            c.lora, c.shift_mu, c.w_decay2 = m.lora, vec(lw.get("shift_mu")), mat(lw.get("w_decay2"))
+            c.decay0, c.bonus = vec(lw.get("decay0")), vec(lw.get("bonus"))
+            if m.moe is not None:
+                e, ew = m.moe, lw["moe"]
+                mc = HybridMoEC(e.experts, e.identity, e.top, e.ff, e.shared_ff, e.limit, e.shared_limit, e.act_alpha,
+                                vec(ew["router"]), vec(ew.get("correction")), mat(ew.get("w_gate_up")), mat(ew.get("w_down")),
+                                mat(ew.get("shared_gate_up")), mat(ew.get("shared_down")))
+                self._moes.append(mc)
+                c.moe = ctypes.pointer(mc)
+
+        for i, (m, lw) in enumerate(zip(cfg.layers, weights["layers"])):
+            fill(larr[i], m, lw, i)
+        for j, (i, sm) in enumerate(sides):
+            # the sibling's record: its own mixer tensors; norms, block form and feed-forward are the primary layer's business
+            fill(larr[len(cfg.layers) + j], sm, dict(weights["layers"][i]["side"], norm1=weights["layers"][i]["norm1"]), i)
+            larr[i].sibling = len(cfg.layers) + j
         runs = cfg.runs()
         rarr = (HybridRunC * len(runs))()
         self.caches, self.pools, self.states = [], [], []
+
+        def storage(m):
+            """(cache, pool, state) of one mixer of one run."""
+            if m.kind in ATTENTION_KINDS:
+                kv = torch.zeros(max_pages * page_size * m.kv_heads * (m.dim + m.vdim), dtype=dtype, device=dev)
+                self.caches.append(kv)
+                if m.kind == "attention":
+                    pool = torch.zeros(max_pages, (page_size - 1) // m.pool + 1, m.kv_heads, m.dim + m.vdim, dtype=torch.float32, device=dev)
+                    self.pools.append(pool)
+                    return kv.data_ptr(), pool.data_ptr(), None
+                return kv.data_ptr(), None, None
+            st = torch.zeros(self.state_slots, m.state_floats(W), dtype=torch.float32, device=dev)
+            self.states.append(st)
+            return None, None, st.data_ptr()
+
         for j, (li, loop_in) in enumerate(runs):
             m = cfg.layers[li]
             rarr[j].layer, rarr[j].loop_in = li, int(loop_in)
-            if m.kind == "attention":
-                kv = torch.zeros(max_pages * page_size * m.kv_heads * (m.dim + m.vdim), dtype=dtype, device=dev)
-                pool = torch.zeros(max_pages, (page_size - 1) // m.pool + 1, m.kv_heads, m.dim + m.vdim, dtype=torch.float32, device=dev)
-                self.caches.append(kv); self.pools.append(pool)
-                rarr[j].cache, rarr[j].pool = kv.data_ptr(), pool.data_ptr()
-            else:
-                per = m.dim * m.vdim + (m.dim + 1 if m.kind == "mlstm" else 0)
-                st = torch.zeros(self.state_slots, m.heads, per, dtype=torch.float32, device=dev)
-                self.states.append(st)
-                rarr[j].state = st.data_ptr()
+            rarr[j].cache, rarr[j].pool, rarr[j].state = storage(m)
+            if m.side is not None:
+                rarr[j].side_cache, rarr[j].side_pool, rarr[j].side_state = storage(m.side)
         self.n_runs = len(runs)
-        cc = HybridConfigC(W, cfg.vocab, len(cfg.layers), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
-                           max_batch, self.max_out, max_pages, max_seq_len, cfg.eps)
+        cc = HybridConfigC(W, cfg.vocab, len(larr), len(runs), 0 if dtype == torch.bfloat16 else 1, page_size, self.max_rows,
+                           max_batch, self.max_out, max_pages, max_seq_len, cfg.eps, NORM_KINDS[cfg.norm_kind], cfg.norm_groups,
+                           cfg.embed_scale)
         cw = HybridWeightsC(ctypes.cast(larr, ctypes.POINTER(HybridLayerC)), ctypes.cast(rarr, ctypes.POINTER(HybridRunC)),
                             mat(weights["embedding"]), mat(weights.get("loop_in")), mat(weights["head"]), vec(weights["final_norm"]))
         self._larr, self._rarr = larr, rarr

@@ -159,23 +159,36 @@ def _orpheus(model_name, device="cuda:0", weights=None, codec_weights=None, chec
     return OrpheusModel(model_name, weights, codec_weights, config=config, device=device, **kw)
 
 
-@register_model("sirodra")
-def _sirodra(model_name, device="cuda:0", weights=None, checkpoint_dir=None, synthetic=False, config=None, **kw):
-    """Text-only hybrid-mixer LM.  checkpoint_dir: a folder with config.json + model.safetensors; synthetic: random weights for
-    `config` (a HybridCfg)."""
-    from .sirodra import SirodraModel, synth_weights
+def _hybrid_lm(module, cls_name, model_name, device, weights, checkpoint_dir, synthetic, config, kw):
+    """Text-only LMs on the hybrid engine.  checkpoint_dir: a folder with config.json + model.safetensors; synthetic: random weights
+    for `config` (a HybridCfg)."""
+    import importlib
+    mod = importlib.import_module(module, __package__)
+    cls = getattr(mod, cls_name)
     kw.pop("detokenize_interval", None)
     if "max_num_pages" in kw and "max_seq_len" not in kw:
         kw["max_seq_len"] = min(kw["max_num_pages"] * kw.get("page_size", 128), 1 << 16)
     if weights is None and checkpoint_dir is not None:
-        return SirodraModel.from_checkpoint(checkpoint_dir, model_name=model_name, device=device, **kw)
+        return cls.from_checkpoint(checkpoint_dir, model_name=model_name, device=device, **kw)
     if config is None:
         raise FileNotFoundError("no checkpoint_dir given: pass checkpoint_dir=... or config=... with weights / synthetic=True")
     if weights is None:
         if not synthetic:
             raise FileNotFoundError("no checkpoint_dir given (offline box): pass checkpoint_dir=... or synthetic=True")
-        weights = synth_weights(config)
-    return SirodraModel(model_name, weights, config, device=device, **kw)
+        weights = mod.synth_weights(config)
+    return cls(model_name, weights, config, device=device, **kw)
+
+
+@register_model("sirodra")
+def _sirodra(model_name, device="cuda:0", weights=None, checkpoint_dir=None, synthetic=False, config=None, **kw):
+    """Hybrid-mixer LM of HGRN2, mLSTM and pooled-window attention layers."""
+    return _hybrid_lm(".sirodra", "SirodraModel", model_name, device, weights, checkpoint_dir, synthetic, config, kw)
+
+
+@register_model("fusanex")
+def _fusanex(model_name, device="cuda:0", weights=None, checkpoint_dir=None, synthetic=False, config=None, **kw):
+    """Parallel-block LM of gated linear recurrent units, attention beside a decaying matrix state, and routed feed-forwards."""
+    return _hybrid_lm(".fusanex", "FusanexModel", model_name, device, weights, checkpoint_dir, synthetic, config, kw)
 
 
 def load_checkpoint_dir(path: str, device: str = "cuda:0", **kw):

@@ -1,4 +1,4 @@
-"""Helpers of the hybrid-mixer (Sirodra) tests: small configurations, random checkpoints, and a driver that feeds token
+"""Helpers of the hybrid-engine tests (Sirodra, Fusanex): small configurations, random checkpoints, and a driver that feeds token
 portions through ModelWorker the way a serving step does."""
 import math
 
@@ -67,11 +67,15 @@ class Driver:
     """A model + ModelWorker on the GPU; `feed` runs one step of token portions and returns the logits of every fed token."""
 
     def __init__(self, cfg, S, dtype=torch.float32, page_size=8, pages=64, slots=4, max_rows=256, max_batch=4):
-        from vox_serve_amd.model.sirodra import SirodraModel, config_from_dict
+        from vox_serve_amd.model import get_model_class
         from vox_serve_amd.worker.base import ModelWorker
-        self.model = SirodraModel("sirodra-test", S, config_from_dict(cfg), dtype=dtype, max_batch_size=max_batch, page_size=page_size,
-                                  max_num_pages=pages, max_seq_len=pages * page_size, max_prefill_tokens=max_rows,
-                                  max_logit_rows=max_rows + max_batch, state_slots=slots)
+        # the registry entry of the config's architecture builds the model, as for a checkpoint folder
+        from vox_serve_amd.model import fusanex, sirodra
+        mod = {"Sirodra": sirodra, "Fusanex": fusanex}[cfg["architecture"]]
+        self.model = get_model_class(cfg["architecture"])(cfg["architecture"].lower() + "-test", weights=S, config=mod.config_from_dict(cfg),
+                                                          dtype=dtype, max_batch_size=max_batch, page_size=page_size, max_num_pages=pages,
+                                                          max_seq_len=pages * page_size, max_prefill_tokens=max_rows,
+                                                          max_logit_rows=max_rows + max_batch, state_slots=slots)
         self.worker = ModelWorker(model=self.model, max_batch_size=max_batch, max_num_pages=pages, page_size=page_size, greedy=True)
         self.live = {}
 

@@ -52,15 +52,21 @@ def time_steps(fn, steps, warmup):
 
 
 def bench_hybrid(width, blocks, vocab, prompts, batches, ctx, steps, warmup, dev):
-    from vox_serve_amd.engine_hybrid import HybridEngine
     from vox_serve_amd.model.sirodra import pack_weights, synth_weights
     cfg = sirodra_cfg(width, blocks, vocab)
+    return bench_hybrid_cfg(cfg, pack_weights(synth_weights(cfg), cfg), layer_bytes(cfg), prompts, batches, ctx, steps, warmup, dev)
+
+
+def bench_hybrid_cfg(cfg, packed, wbytes, prompts, batches, ctx, steps, warmup, dev):
+    """Any design of the hybrid engine: `packed` = the engine's weight layout, wbytes = weight bytes a one-row decode step streams."""
+    from vox_serve_amd.engine_hybrid import HybridEngine
+    vocab = cfg.vocab
     ps = 128
     maxp, maxb = max(prompts), max(batches)
     pages = max((maxp + ps - 1) // ps, maxb * ((ctx + 64 + ps - 1) // ps)) + 1
-    eng = HybridEngine(cfg, pack_weights(synth_weights(cfg), cfg), dtype=torch.bfloat16, max_batch=maxb, page_size=ps, max_pages=pages,
+    eng = HybridEngine(cfg, packed, dtype=torch.bfloat16, max_batch=maxb, page_size=ps, max_pages=pages,
                        max_seq_len=max(maxp, ctx + 64) + ps, max_prefill_rows=maxp, state_slots=maxb, device=dev)
-    out = {"weight_bytes_per_step": layer_bytes(cfg), "prefill": {}, "decode": {}}
+    out = {"weight_bytes_per_step": wbytes, "prefill": {}, "decode": {}}
     sc = eng.sampling_cfg(greedy=True)
     rng = np.random.default_rng(0)
     for n in prompts:
@@ -86,7 +92,7 @@ def bench_hybrid(width, blocks, vocab, prompts, batches, ctx, steps, warmup, dev
             eng.frame(B, max(kv), sc, feedback=True)
         dt = time_steps(step, steps, warmup)
         kv[:] = [ctx] * B
-        out["decode"][str(B)] = {"ms": dt * 1e3, "tokens_per_s": B / dt, "weight_GBps": layer_bytes(cfg) / dt / 1e9}
+        out["decode"][str(B)] = {"ms": dt * 1e3, "tokens_per_s": B / dt, "weight_GBps": wbytes / dt / 1e9}
     eng.close()
     return out
 

@@ -55,14 +55,17 @@ template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float a
 __device__ __forceinline__ float hb_gelu_tanh(float z) {
     return 0.5f * z * (1.0f + tanhf(0.79788456080286535588f * (z + 0.044715f * z * z * z)));
 }
-// A tile GEMM over a gathered subset of rows (routed experts): block z multiplies the rows list[z*cap + 0 .. count[z]) with the
-// z-th matrix (w_stride elements apart); the A row of list entry v is v / a_div, its C row is v.  count == NULL: plain GEMM.
+// Several products in one launch: product z uses the matrix Wt + z*w_stride, the activations A + z*a_stride, the outputs
+// C + z*c_stride and the bias + z*b_stride (a strided batch: block-diagonal matrices, projections that each read their own input).
+// count != NULL (routed experts): product z takes the gathered rows list[z*cap + 0 .. count[z]); the A row of list entry v is
+// v / a_div, its C row is v.
 struct hb_rowmap {
     const int* count;
     const int* list;
     int cap, a_div;
-    long w_stride;
+    long w_stride, a_stride, c_stride, b_stride;
 };
+static inline hb_rowmap hb_plain() { return hb_rowmap{nullptr, nullptr, 0, 1, 0, 0, 0, 0}; }
 
 // ---- embedding gather: x[row] = table[id]; the second half of both residual buffers keeps the embedding output ----------
 template <typename T>
@@ -174,11 +177,14 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
     const int tid = threadIdx.x, lane = tid & 63, wv = tid >> 6;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
     const int* lst = nullptr;
+    Wt += (size_t)blockIdx.z * rm.w_stride;
+    A += (size_t)blockIdx.z * rm.a_stride;
+    C += (size_t)blockIdx.z * rm.c_stride;
+    if (bias) bias += (size_t)blockIdx.z * rm.b_stride;
     if (rm.count) {
         M = rm.count[blockIdx.z];
         if (m0 >= M) return;
         lst = rm.list + (size_t)blockIdx.z * rm.cap;
-        Wt += (size_t)blockIdx.z * rm.w_stride;
     }
     constexpr int MT = BM == 64 ? 2 : 1, NT = BM == 64 ? 2 : 1;
     const int mt0 = BM == 64 ? (wv >> 1) * 2 : 0, nt0 = BM == 64 ? (wv & 1) * 2 : wv;
@@ -277,11 +283,14 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
     const int tid = threadIdx.x, tx = tid & 15, ty = tid >> 4;
     const int m0 = blockIdx.y * BM, n0 = blockIdx.x * 64;
     const int* lst = nullptr;
+    Wt += (size_t)blockIdx.z * rm.w_stride;
+    A += (size_t)blockIdx.z * rm.a_stride;
+    C += (size_t)blockIdx.z * rm.c_stride;
+    if (bias) bias += (size_t)blockIdx.z * rm.b_stride;
     if (rm.count) {
         M = rm.count[blockIdx.z];
         if (m0 >= M) return;
         lst = rm.list + (size_t)blockIdx.z * rm.cap;
-        Wt += (size_t)blockIdx.z * rm.w_stride;
     }
     for (int r = tid; r < BM; r += 256) arow[r] = m0 + r < M ? (lst ? lst[m0 + r] : m0 + r) : -1;
     __syncthreads();
@@ -332,9 +341,13 @@ __global__ __launch_bounds__(256) void k_hb_gemm_f32(const float* A, long lda, c
 // the activations; lanes own k-chunks c, c + 64, ...; butterfly at the end.  The order of each output's sum depends on K only.
 template <typename T, int MR, int EPI, int HB_GEMV_CPW>
 __global__ __launch_bounds__(256) void k_hb_gemv(const float* A, long lda, const T* Wt, const float* bias, float* C, long ldc, int M, int N,
-                                                 int K) {
+                                                 int K, hb_rowmap rm) {
     const int lane = threadIdx.x & 63, n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * HB_GEMV_CPW;
     if (n0 >= N) return;
+    Wt += (size_t)blockIdx.y * rm.w_stride;
+    A += (size_t)blockIdx.y * rm.a_stride;
+    C += (size_t)blockIdx.y * rm.c_stride;
+    if (bias) bias += (size_t)blockIdx.y * rm.b_stride;
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
     float acc[MR][HB_GEMV_CPW];
 #pragma unroll
@@ -487,8 +500,12 @@ bool hb_try_ln_gemv(hipStream_t st, int epi, const float* X, long ldx, const int
 // converted to bf16 in registers); the eight partial tiles are added in wave order.  Needs K % 32 == 0.
 template <int EPI>
 __global__ __launch_bounds__(512) void k_hb_gemm_rows16(const float* A, long lda, const bf16_t* Wt, const float* bias, float* C, long ldc, int M,
-                                                        int N, int K) {
+                                                        int N, int K, hb_rowmap rm) {
     __shared__ float red[8][16][17];
+    Wt += (size_t)blockIdx.y * rm.w_stride;
+    A += (size_t)blockIdx.y * rm.a_stride;
+    C += (size_t)blockIdx.y * rm.c_stride;
+    if (bias) bias += (size_t)blockIdx.y * rm.b_stride;
     const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int n0 = blockIdx.x * 16, col = lane & 15, kb = lane >> 4;
     const int nsteps = K >> 5;
@@ -531,59 +548,64 @@ __global__ __launch_bounds__(512) void k_hb_gemm_rows16(const float* A, long lda
         }
     }
 }
+// every operand of every product of a strided batch is 16-byte aligned
+static inline bool hb_batch_aligned(const hb_rowmap& rm, int nz, size_t wsize) {
+    return nz == 1 || ((rm.w_stride * wsize) % 16 == 0 && (rm.a_stride * 4) % 16 == 0);
+}
 template <int EPI>
-bool hb_try_rows16(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K) {
-    if (M < 2 || M > 16 || (K & 31) || (lda & 3) || ((size_t)A & 15) || ((size_t)W & 15)) return false;
-    hipLaunchKernelGGL((k_hb_gemm_rows16<EPI>), dim3((N + 15) / 16), dim3(512), 0, st, A, lda, W, bias, C, ldc, M, N, K);
+bool hb_try_rows16(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K,
+                   const hb_rowmap& rm, int nz) {
+    if (M < 2 || M > 16 || (K & 31) || (lda & 3) || ((size_t)A & 15) || ((size_t)W & 15) || !hb_batch_aligned(rm, nz, 2)) return false;
+    hipLaunchKernelGGL((k_hb_gemm_rows16<EPI>), dim3((N + 15) / 16, nz), dim3(512), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     return true;
 }
 template <int EPI>
-bool hb_try_rows16(hipStream_t, const float*, long, const float*, const float*, float*, long, int, int, int) { return false; }
-
-template <typename T, int EPI>
-int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K);
+bool hb_try_rows16(hipStream_t, const float*, long, const float*, const float*, float*, long, int, int, int, const hb_rowmap&, int) { return false; }
 
 // rm.count != NULL: `groups` gathered GEMMs of at most M rows each in one launch (see hb_rowmap)
 template <int EPI>
 int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const bf16_t* W, const float* bias, float* C, long ldc, int M, int N, int K,
-                  hb_rowmap rm = hb_rowmap{nullptr, nullptr, 0, 1, 0}, int groups = 1) {
+                  hb_rowmap rm = hb_plain(), int groups = 1) {
     if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_bf16<16, EPI>), dim3((N + 63) / 64, 1, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     else hipLaunchKernelGGL((k_hb_gemm_bf16<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     return VOX_OK;
 }
 template <int EPI>
 int hb_gemm_tiles(hipStream_t st, const float* A, long lda, const float* W, const float* bias, float* C, long ldc, int M, int N, int K,
-                  hb_rowmap rm = hb_rowmap{nullptr, nullptr, 0, 1, 0}, int groups = 1) {
+                  hb_rowmap rm = hb_plain(), int groups = 1) {
     if (M <= 16) hipLaunchKernelGGL((k_hb_gemm_f32<16, EPI>), dim3((N + 63) / 64, 1, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     else hipLaunchKernelGGL((k_hb_gemm_f32<64, EPI>), dim3((N + 63) / 64, (M + 63) / 64, groups), dim3(256), 0, st, A, lda, W, bias, C, ldc, M, N, K, rm);
     return VOX_OK;
 }
+// nz > 1: a strided batch of nz products (rm gives the strides) in one launch
 template <typename T, int EPI>
-int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
+int hb_gemm_epi(hipStream_t st, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K,
+                const hb_rowmap& rm, int nz) {
     if (M <= 0 || N <= 0) return VOX_OK;
     // four columns per wave once that still leaves a block for every compute unit several times over
     const bool wide = N >= 16 * 1024;
-    const dim3 g(wide ? (N + 15) / 16 : (N + 3) / 4), b(256);
+    const dim3 g(wide ? (N + 15) / 16 : (N + 3) / 4, nz), b(256);
 #define HB_GEMV(MR_) \
     do { \
-        if (wide) hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 4>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K); \
-        else hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 1>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K); \
+        if (wide) hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 4>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K, rm); \
+        else hipLaunchKernelGGL((k_hb_gemv<T, MR_, EPI, 1>), g, b, 0, st, A, lda, W, bias, C, ldc, M, N, K, rm); \
     } while (0)
-    if (hb_try_rows16<EPI>(st, A, lda, W, bias, C, ldc, M, N, K)) {}
+    if (hb_try_rows16<EPI>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz)) {}
     else if (M == 1) HB_GEMV(1);
     else if (M == 2) HB_GEMV(2);
     else if (M <= 4) HB_GEMV(4);
     else if (M <= 8) HB_GEMV(8);
 #undef HB_GEMV
-    else return hb_gemm_tiles<EPI>(st, A, lda, W, bias, C, ldc, M, N, K);
+    else return hb_gemm_tiles<EPI>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
     return VOX_OK;
 }
 template <typename T>
-int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K) {
-    if (epi == HB_EPI_GELU) return hb_gemm_epi<T, HB_EPI_GELU>(st, A, lda, W, bias, C, ldc, M, N, K);
-    if (epi == HB_EPI_RESID) return hb_gemm_epi<T, HB_EPI_RESID>(st, A, lda, W, bias, C, ldc, M, N, K);
-    if (epi == HB_EPI_TANH) return hb_gemm_epi<T, HB_EPI_TANH>(st, A, lda, W, bias, C, ldc, M, N, K);
-    return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K);
+int hb_gemm(hipStream_t st, int epi, const float* A, long lda, const T* W, const float* bias, float* C, long ldc, int M, int N, int K,
+            const hb_rowmap& rm = hb_plain(), int nz = 1) {
+    if (epi == HB_EPI_GELU) return hb_gemm_epi<T, HB_EPI_GELU>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
+    if (epi == HB_EPI_RESID) return hb_gemm_epi<T, HB_EPI_RESID>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
+    if (epi == HB_EPI_TANH) return hb_gemm_epi<T, HB_EPI_TANH>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
+    return hb_gemm_epi<T, HB_EPI_STORE>(st, A, lda, W, bias, C, ldc, M, N, K, rm, nz);
 }
 
 // ---- linear recurrences ------------------------------------------------------------------------------------------------------
@@ -844,6 +866,71 @@ __global__ __launch_bounds__(64) void k_hb_rglru_scan(const float* proj, long ld
         else if (q >= 0) v = st[(size_t)(1 + i + n) * C + c];
         st[(size_t)(1 + i) * C + c] = v;
     }
+}
+
+// Long portions: the same recurrence with the request's rows cut into 32 chunks that run side by side.  Block = 32 channels x 32
+// chunks.  Pass 1: every thread evaluates the gates of its chunk (a and b = sqrt(1 - a^2) i u replace the gate pre-activations in
+// proj) and reduces the chunk to S_out = A S_in + B.  Pass 2: the carry into chunk k is the slot's state pushed through chunks
+// 0 .. k-1 in order.  Pass 3: the chunk is replayed from its carry with the recurrence itself and the outputs are written.
+#define HB_LRU_CHUNKS 32
+__global__ __launch_bounds__(1024) void k_hb_rglru_scan_chunked(float* proj, long ldp, float* out, long ldo, const float* lam, float* state,
+                                                                const int* req_rows, const int* req_state, const int* pos, int C, int bs,
+                                                                int taps, float rec_scale, float out_scale) {
+    __shared__ float sA[HB_LRU_CHUNKS][32], sB[HB_LRU_CHUNKS][32];
+    const int r = blockIdx.x, cl = threadIdx.x & 31, k = threadIdx.x >> 5, c = blockIdx.y * 32 + cl;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const bool ok = c < C;
+    const int cc = ok ? c : C - 1;
+    const int n = re - rs, len = (n + HB_LRU_CHUNKS - 1) / HB_LRU_CHUNKS;
+    const int tb = rs + k * len < re ? rs + k * len : re, te = tb + len < re ? tb + len : re;
+    float* st = state + (size_t)req_state[r] * taps * C;
+    const int p0 = pos[rs];
+    const float lv = lam[cc];
+    const float sp = lv > 20.f ? lv : log1pf(expf(lv));
+    const int blk = cc / bs, j = cc - blk * bs;
+    const size_t off_r = (size_t)3 * C + (size_t)blk * 2 * bs + j, off_i = off_r + bs;
+    float A = 1.f, B = 0.f;
+    for (int t0 = tb; t0 < te; t0 += 4) {
+        float a[4], b[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int t = t0 + q < te ? t0 + q : te - 1;
+            const float* pr = proj + (size_t)t * ldp;
+            const float rg = hb_sigmoid(pr[off_r]), ig = hb_sigmoid(pr[off_i]);
+            a[q] = expf(-rec_scale * rg * sp);
+            b[q] = sqrtf(1.0f - a[q] * a[q]) * (ig * pr[2 * C + cc]);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+            if (t0 + q < te) {
+                float* pr = proj + (size_t)(t0 + q) * ldp;
+                if (ok) { pr[off_r] = a[q]; pr[off_i] = b[q]; }
+                B = a[q] * B + b[q];
+                A *= a[q];
+            }
+    }
+    sA[k][cl] = A;
+    sB[k][cl] = B;
+    __syncthreads();
+    float S = p0 == 0 ? 0.f : st[cc];
+    for (int q = 0; q < k; ++q) S = sA[q][cl] * S + sB[q][cl];
+    for (int t = tb; t < te; ++t) {
+        const float* pr = proj + (size_t)t * ldp;
+        S = pr[off_r] * S + pr[off_i];
+        if (ok) out[(size_t)t * ldo + c] = S * hb_gelu_tanh(pr[cc]) * out_scale;
+    }
+    if (!ok) return;
+    // chunks behind the portion's end are empty (A = 1, B = 0): the last thread of a channel holds the final state
+    if (k == HB_LRU_CHUNKS - 1) st[c] = S;
+    if (k == 0)
+        for (int i = 0; i < taps - 1; ++i) {
+            const int q = p0 + n - (taps - 1) + i;
+            float v = 0.f;
+            if (q >= p0) v = proj[(size_t)(rs + q - p0) * ldp + C + c];
+            else if (q >= 0) v = st[(size_t)(1 + i + n) * C + c];
+            st[(size_t)(1 + i) * C + c] = v;
+        }
 }
 
 // ---- matrix-state recurrence with token shift and a data-dependent decay per key channel ------------------------------------
@@ -1385,21 +1472,53 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
 }
 
 // ---- routed feed-forward --------------------------------------------------------------------------------------------------
-// One wave per row: s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first index
-// wins a tie) in descending order; weights = their s / (sum + 1e-20).  sel[row*top + k] = router output index, wgt likewise.
-__global__ __launch_bounds__(64) void k_hb_moe_route(const float* z, const float* corr, int nE, int top, int* sel, float* wgt) {
+// One wave per row: router logits z_j = router[j] . h in fp32 (lane-strided sums and a butterfly: an order fixed by the width, the
+// same for every step shape), s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first
+// index wins a tie) in descending order; weights = their s / (sum + 1e-20).  sel[row*top + k] = router output index, wgt likewise.
+__global__ __launch_bounds__(64) void k_hb_moe_router(const float* h, long ldh, const float* router, const float* corr, int W, int nE, int top,
+                                                      int* sel, float* wgt) {
     extern __shared__ float sm[];
-    float* sc = sm;                    // [nE] scores
+    float* sc = sm;                    // [nE] logits, then scores
     float* ch = sm + nE;               // [nE] choice values
     int* pick = (int*)(sm + 2 * nE);   // [top]
     const int row = blockIdx.x, lane = threadIdx.x;
-    const float* zr = z + (size_t)row * nE;
+    const float* x = h + (size_t)row * ldh;
+    const bool vec = (W % 4 == 0) && (ldh % 4 == 0) && ((((size_t)h) & 15) == 0) && ((((size_t)router) & 15) == 0);
+    for (int j0 = 0; j0 < nE; j0 += 4) {
+        float acc[4] = {0.f, 0.f, 0.f, 0.f};
+        const float* r[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) r[j] = router + (size_t)(j0 + j < nE ? j0 + j : nE - 1) * W;
+        if (vec) {
+            for (int k = lane * 4; k < W; k += 256) {
+                const float4 xv = *(const float4*)(x + k);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {
+                    const float4 rv = *(const float4*)(r[j] + k);
+                    acc[j] = fmaf(rv.x, xv.x, acc[j]); acc[j] = fmaf(rv.y, xv.y, acc[j]);
+                    acc[j] = fmaf(rv.z, xv.z, acc[j]); acc[j] = fmaf(rv.w, xv.w, acc[j]);
+                }
+            }
+        } else {
+            for (int k = lane; k < W; k += 64) {
+                const float xv = x[k];
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[j] = fmaf(r[j][k], xv, acc[j]);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const float v = hb_wave_sum(acc[j]);
+            if (lane == 0 && j0 + j < nE) sc[j0 + j] = v;
+        }
+    }
+    __syncthreads();
     float mx = -INFINITY;
-    for (int i = lane; i < nE; i += 64) mx = fmaxf(mx, zr[i]);
+    for (int i = lane; i < nE; i += 64) mx = fmaxf(mx, sc[i]);
     mx = hb_wave_max(mx);
     float sum = 0.f;
     for (int i = lane; i < nE; i += 64) {
-        const float e = expf(zr[i] - mx);
+        const float e = expf(sc[i] - mx);
         sc[i] = e;
         sum += e;
     }
@@ -1470,65 +1589,92 @@ __global__ __launch_bounds__(256) void k_hb_glu_clamp(const float* gu, float* y,
         y[(size_t)row * ff + j] = g * hb_sigmoid(alpha * g) * (u + 1.0f);
     }
 }
-// Few-row steps: one routed entry per blockIdx.y, a wave per output column (the order of k_hb_gemv's sum).  A row = entry / a_div,
-// the matrix is the entry's expert's; entries of identity outputs are skipped.  GLU: the wave takes the gate row n and the up row
-// ff + n and stores the activated value (N = ff output columns); else a plain product with N columns.
-template <typename T, bool GLU>
-__global__ __launch_bounds__(256) void k_hb_moe_gemv(const float* A, long lda, int a_div, const T* Wt, long w_stride, const int* sel, int experts,
-                                                     float* C, long ldc, int N, int K, float limit, float alpha) {
-    const int entry = blockIdx.y, lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
-    const int e = sel[entry];
-    if (n >= N || e >= experts) return;
-    const float* xr = A + (size_t)(entry / a_div) * lda;
-    const T* w0 = Wt + (size_t)e * w_stride + (size_t)n * K;
-    const T* w1 = w0 + (size_t)N * K;
+// Few-row steps.  Entries per row: its `top` routed choices, then (shared_ff > 0) the shared expert.
+// A lane-chunked dot product in k_hb_gemv's order: chunks of CH at lane*CH + 64*CH*i, then a butterfly.
+template <typename T>
+__device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, bool vec, int lane) {
     constexpr int CH = sizeof(T) == 2 ? 8 : 4;
-    float a0 = 0.f, a1 = 0.f;
-    const bool vec = (K % CH == 0) && ((((size_t)Wt) & 15) == 0) && ((w_stride * sizeof(T)) % 16 == 0) && (lda % 4 == 0) && ((((size_t)A) & 15) == 0);
+    float a = 0.f;
     if (vec) {
         for (int k = lane * CH; k < K; k += 64 * CH) {
-            float wa[CH], wb[CH];
+            float wv[CH];
             if (sizeof(T) == 2) {
-                const uint4 u = *(const uint4*)(w0 + k);
-                wa[0] = bflo(u.x); wa[1] = bfhi(u.x); wa[2] = bflo(u.y); wa[3] = bfhi(u.y);
-                if (CH == 8) { wa[4] = bflo(u.z); wa[5] = bfhi(u.z); wa[6] = bflo(u.w); wa[7] = bfhi(u.w); }
-                if (GLU) {
-                    const uint4 u2 = *(const uint4*)(w1 + k);
-                    wb[0] = bflo(u2.x); wb[1] = bfhi(u2.x); wb[2] = bflo(u2.y); wb[3] = bfhi(u2.y);
-                    if (CH == 8) { wb[4] = bflo(u2.z); wb[5] = bfhi(u2.z); wb[6] = bflo(u2.w); wb[7] = bfhi(u2.w); }
-                }
+                const uint4 u = *(const uint4*)(w + k);
+                wv[0] = bflo(u.x); wv[1] = bfhi(u.x); wv[2] = bflo(u.y); wv[3] = bfhi(u.y);
+                if (CH == 8) { wv[4] = bflo(u.z); wv[5] = bfhi(u.z); wv[6] = bflo(u.w); wv[7] = bfhi(u.w); }
             } else {
-                const float4 u = *(const float4*)(w0 + k);
-                wa[0] = u.x; wa[1] = u.y; wa[2] = u.z; wa[3] = u.w;
-                if (GLU) {
-                    const float4 u2 = *(const float4*)(w1 + k);
-                    wb[0] = u2.x; wb[1] = u2.y; wb[2] = u2.z; wb[3] = u2.w;
-                }
+                const float4 u = *(const float4*)(w + k);
+                wv[0] = u.x; wv[1] = u.y; wv[2] = u.z; wv[3] = u.w;
             }
 #pragma unroll
-            for (int i = 0; i < CH; ++i) {
-                const float x = hb_operand<T>(xr[k + i]);
-                a0 = fmaf(wa[i], x, a0);
-                if (GLU) a1 = fmaf(wb[i], x, a1);
-            }
+            for (int i = 0; i < CH; ++i) a = fmaf(wv[i], hb_operand<T>(x[k + i]), a);
         }
     } else {
-        for (int k = lane; k < K; k += 64) {
-            const float x = hb_operand<T>(xr[k]);
-            a0 = fmaf(hb_ld(w0 + k), x, a0);
-            if (GLU) a1 = fmaf(hb_ld(w1 + k), x, a1);
-        }
+        for (int k = lane; k < K; k += 64) a = fmaf(hb_ld(w + k), hb_operand<T>(x[k]), a);
     }
-    a0 = hb_wave_sum(a0);
-    if (GLU) a1 = hb_wave_sum(a1);
+    return hb_wave_sum(a);
+}
+struct hb_moe_small {
+    const int* sel;
+    const float* wgt;
+    int top, experts, ff, shared_ff, ld_act;
+    float limit, shared_limit, alpha;
+};
+// gate / up products + activation of every entry: block (column tile, entry); a wave takes gate row n and up row ff + n of the
+// entry's expert and stores g * sigmoid(alpha g) * (u + 1) with the clamps of that expert.  act row of an entry: ld_act floats.
+template <typename T>
+__global__ __launch_bounds__(256) void k_hb_moe_gate_up(const float* h, long ldh, const T* w_gate_up, const T* shared_gate_up, float* act, int W,
+                                                        hb_moe_small q) {
+    const int per = q.top + (q.shared_ff > 0 ? 1 : 0);
+    const int entry = blockIdx.y, row = entry / per, slot = entry - row * per, lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    const T* wg;
+    int N;
+    float limit;
+    if (slot < q.top) {
+        const int e = q.sel[(size_t)row * q.top + slot];
+        if (e >= q.experts) return;
+        wg = w_gate_up + (size_t)e * 2 * q.ff * W;
+        N = q.ff;
+        limit = q.limit;
+    } else {
+        wg = shared_gate_up;
+        N = q.shared_ff;
+        limit = q.shared_limit;
+    }
+    if (n >= N) return;
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    const float* x = h + (size_t)row * ldh;
+    const bool vec = (W % CH == 0) && ((((size_t)wg) & 15) == 0) && (ldh % 4 == 0) && ((((size_t)h) & 15) == 0);
+    const float g0 = hb_dot_wave<T>(wg + (size_t)n * W, x, W, vec, lane), u0 = hb_dot_wave<T>(wg + (size_t)(N + n) * W, x, W, vec, lane);
     if (lane == 0) {
-        if (GLU) {
-            const float g = fminf(a0, limit), u = fminf(fmaxf(a1, -limit), limit);
-            C[(size_t)entry * ldc + n] = g * hb_sigmoid(alpha * g) * (u + 1.0f);
-        } else {
-            C[(size_t)entry * ldc + n] = a0;
-        }
+        const float g = fminf(g0, limit), u = fminf(fmaxf(u0, -limit), limit);
+        act[(size_t)entry * q.ld_act + n] = g * hb_sigmoid(q.alpha * g) * (u + 1.0f);
     }
+}
+// down products of a row's entries, weighted and added to the residual stream: a wave per (row, output column):
+// x[row][c] += sum_k wgt_k * (identity ? h[row][c] : down_{e_k}[c] . act_k)  +  shared_down[c] . act_shared, k ascending.
+template <typename T>
+__global__ __launch_bounds__(256) void k_hb_moe_down_combine(const float* h, long ldh, const T* w_down, const T* shared_down, const float* act,
+                                                             float* x, long ldx, int W, hb_moe_small q) {
+    const int per = q.top + (q.shared_ff > 0 ? 1 : 0);
+    const int row = blockIdx.y, lane = threadIdx.x & 63, c = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (c >= W) return;
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    const bool avec = (q.ld_act % 4 == 0) && ((((size_t)act) & 15) == 0);
+    float acc = 0.f;
+    for (int k = 0; k < q.top; ++k) {
+        const int e = q.sel[(size_t)row * q.top + k];
+        const float wk = q.wgt[(size_t)row * q.top + k];
+        if (e >= q.experts) { acc = fmaf(wk, h[(size_t)row * ldh + c], acc); continue; }
+        const T* wd = w_down + ((size_t)e * W + c) * q.ff;
+        const bool vec = avec && (q.ff % CH == 0) && ((((size_t)w_down) & 15) == 0);
+        acc = fmaf(wk, hb_dot_wave<T>(wd, act + (size_t)(row * per + k) * q.ld_act, q.ff, vec, lane), acc);
+    }
+    if (q.shared_ff > 0) {
+        const bool vec = avec && (q.shared_ff % CH == 0) && ((((size_t)shared_down) & 15) == 0);
+        acc += hb_dot_wave<T>(shared_down + (size_t)c * q.shared_ff, act + (size_t)(row * per + q.top) * q.ld_act, q.shared_ff, vec, lane);
+    }
+    if (lane == 0) x[(size_t)row * ldx + c] += acc;
 }
 // x[row] += sum_k wgt[row*top + k] * (identity output ? h[row] : expert_out[row*top + k]), k ascending
 __global__ __launch_bounds__(256) void k_hb_moe_combine(float* x, long ldx, const float* h, long ldh, const float* eo, const int* sel,
@@ -1586,6 +1732,9 @@ __global__ void k_hb_feedback(const int* out_ids, int* input_ids, uint64_t* rng,
 
 }  // namespace
 
+#define HB_MOE_GEMV_ROWS 8    // steps of at most this many rows run the routed feed-forward entry by entry
+#define HB_LRU_SEQ_ROWS 64    // steps of at most this many rows run the gated linear recurrent unit token by token
+
 struct vox_hybrid {
     vox_ctx* ctx;
     vox_hybrid_config cfg;
@@ -1595,7 +1744,7 @@ struct vox_hybrid {
     vox_hybrid_weights w;
     float *xa = nullptr, *xb = nullptr, *h = nullptr, *h2 = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
     float *shift = nullptr;                 // [5][max_rows][width]: token-shift mixes
-    float *moe_z = nullptr, *moe_wgt = nullptr, *moe_act = nullptr, *moe_out = nullptr;
+    float *moe_wgt = nullptr, *moe_act = nullptr, *moe_out = nullptr;
     int *moe_sel = nullptr, *moe_list = nullptr, *moe_count = nullptr;
     bf16_t* logits16 = nullptr;
     float* attn_ws = nullptr;
@@ -1657,9 +1806,9 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         hipLaunchKernelGGL(k_hb_shift_mix, dim3(n), dim3(256), 0, st, hn, (long)W, L.shift_mu, m->shift, rows_stride, state, per_slot,
                            (long)HD * L.dim, io->pos, io->row_req, io->req_rows, io->req_state, W);
         const T* wi = (const T*)L.w_in;
-        for (int s2 = 0; s2 < 4; ++s2)
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->shift + s2 * rows_stride, W, wi + (size_t)s2 * HD * W, L.b_in ? L.b_in + s2 * HD : nullptr,
-                               m->proj + s2 * HD, n_proj, n, HD, W));
+        // r, k, v, g: four products of one shape, each on its own mix, in one launch
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->shift, W, wi, L.b_in, m->proj, n_proj, n, HD, W,
+                           hb_rowmap{nullptr, nullptr, 0, 1, (long)HD * W, rows_stride, (long)HD, (long)HD}, 4));
         VOX_TRY(hb_gemm<T>(st, HB_EPI_TANH, m->shift + 4 * rows_stride, W, wi + (size_t)4 * HD * W, nullptr, m->proj + 4 * HD, n_proj, n, L.lora, W));
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + 4 * HD, n_proj, (const T*)L.w_decay2, L.decay0, m->proj + 4 * HD + L.lora, n_proj, n, HD, L.lora));
         const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
@@ -1704,11 +1853,16 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         hipLaunchKernelGGL(k_hb_conv_causal, dim3(n, (C + 255) / 256), dim3(256), 0, st, m->proj, (long)n_proj, L.conv_w, L.conv_b, state, io->pos,
                            io->row_req, io->req_rows, io->req_state, C, L.conv_taps);
         // block-diagonal gates: block b's 2*bs outputs (r rows, then i rows) from its bs channels of the convolution's output
-        for (int b = 0; b < L.heads; ++b)
-            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + 2 * C + b * bs, n_proj, (const T*)L.w_gates + (size_t)b * 2 * bs * bs,
-                               L.b_gates ? L.b_gates + (size_t)b * 2 * bs : nullptr, m->proj + 3 * C + (size_t)b * 2 * bs, n_proj, n, 2 * bs, bs));
-        hipLaunchKernelGGL(k_hb_rglru_scan, dim3(n_req, (C + 63) / 64), dim3(64), 0, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.lam, state,
-                           io->req_rows, io->req_state, io->pos, C, bs, L.conv_taps, L.rec_scale, L.out_scale);
+        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + 2 * C, n_proj, (const T*)L.w_gates, L.b_gates, m->proj + 3 * C, n_proj, n, 2 * bs, bs,
+                           hb_rowmap{nullptr, nullptr, 0, 1, (long)2 * bs * bs, (long)bs, (long)2 * bs, (long)2 * bs}, L.heads));
+        // steps of many rows cut every request's rows into chunks that run side by side; the chunked form replays the same recurrence
+        // from carries that were pushed through whole chunks, which differs from the plain form by rounding only
+        if (n > HB_LRU_SEQ_ROWS)
+            hipLaunchKernelGGL(k_hb_rglru_scan_chunked, dim3(n_req, (C + 31) / 32), dim3(1024), 0, st, m->proj, (long)n_proj, m->mix, (long)n_mix,
+                               L.lam, state, io->req_rows, io->req_state, io->pos, C, bs, L.conv_taps, L.rec_scale, L.out_scale);
+        else
+            hipLaunchKernelGGL(k_hb_rglru_scan, dim3(n_req, (C + 63) / 64), dim3(64), 0, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.lam, state,
+                               io->req_rows, io->req_state, io->pos, C, bs, L.conv_taps, L.rec_scale, L.out_scale);
     } else {
         const bool causal = L.kind == VOX_MIXER_CAUSAL_ATTN;
         const int H = L.heads, G = L.kv_heads, QG = H / G;
@@ -1745,28 +1899,29 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
 
 // Routed feed-forward of the normed rows h2, added to cur.  Few rows: one GEMV pair per routed entry; more: the entries are
 // listed per expert and every expert multiplies its own rows in one tile launch.
-#define HB_MOE_GEMV_ROWS 8
 template <typename T>
 static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const float* h2, float* cur, long ldx, int n) {
     const int W = m->cfg.width, nE = E.experts + E.identity, top = E.top, ne = n * top, ff = E.ff;
-    VOX_TRY(hb_gemm<float>(st, HB_EPI_STORE, h2, W, E.router, nullptr, m->moe_z, nE, n, nE, W));
-    hipLaunchKernelGGL(k_hb_moe_route, dim3(n), dim3(64), (size_t)(2 * nE + top) * 4, st, m->moe_z, E.correction, nE, top, m->moe_sel, m->moe_wgt);
+    hipLaunchKernelGGL(k_hb_moe_router, dim3(n), dim3(64), (size_t)(2 * nE + top) * 4, st, h2, (long)W, E.router, E.correction, W, nE, top,
+                       m->moe_sel, m->moe_wgt);
+    if (n <= HB_MOE_GEMV_ROWS) {
+        const int per = top + (E.shared_ff > 0 ? 1 : 0), maxf = ff > E.shared_ff ? ff : E.shared_ff;
+        const hb_moe_small q{m->moe_sel, m->moe_wgt, top, E.experts, ff, E.shared_ff, m->max_eff, E.limit, E.shared_limit, E.act_alpha};
+        hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((maxf + 3) / 4, n * per), dim3(256), 0, st, h2, (long)W, (const T*)E.w_gate_up,
+                           (const T*)E.shared_gate_up, m->moe_act, W, q);
+        hipLaunchKernelGGL((k_hb_moe_down_combine<T>), dim3((W + 3) / 4, n), dim3(256), 0, st, h2, (long)W, (const T*)E.w_down,
+                           (const T*)E.shared_down, m->moe_act, cur, ldx, W, q);
+        return VOX_OK;
+    }
     if (E.experts > 0) {
-        if (n <= HB_MOE_GEMV_ROWS) {
-            hipLaunchKernelGGL((k_hb_moe_gemv<T, true>), dim3((ff + 3) / 4, ne), dim3(256), 0, st, h2, (long)W, top, (const T*)E.w_gate_up,
-                               (long)2 * ff * W, m->moe_sel, E.experts, m->moe_act, (long)ff, ff, W, E.limit, E.act_alpha);
-            hipLaunchKernelGGL((k_hb_moe_gemv<T, false>), dim3((W + 3) / 4, ne), dim3(256), 0, st, m->moe_act, (long)ff, 1, (const T*)E.w_down,
-                               (long)W * ff, m->moe_sel, E.experts, m->moe_out, (long)W, W, ff, 0.f, 0.f);
-        } else {
-            const int cap = m->cfg.max_rows;
-            hipLaunchKernelGGL(k_hb_moe_group, dim3(E.experts), dim3(256), 0, st, m->moe_sel, ne, cap, m->moe_list, m->moe_count);
-            VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, h2, (long)W, (const T*)E.w_gate_up, nullptr, m->ff, (long)2 * ff, n, 2 * ff, W,
-                                                hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)2 * ff * W}, E.experts));
-            hipLaunchKernelGGL(k_hb_glu_clamp, dim3(ne, (ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, ff, E.limit, E.act_alpha,
-                               m->moe_sel, E.experts);
-            VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, m->moe_act, (long)ff, (const T*)E.w_down, nullptr, m->moe_out, (long)W, n, W, ff,
-                                                hb_rowmap{m->moe_count, m->moe_list, cap, 1, (long)W * ff}, E.experts));
-        }
+        const int cap = m->cfg.max_rows;
+        hipLaunchKernelGGL(k_hb_moe_group, dim3(E.experts), dim3(256), 0, st, m->moe_sel, ne, cap, m->moe_list, m->moe_count);
+        VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, h2, (long)W, (const T*)E.w_gate_up, nullptr, m->ff, (long)2 * ff, n, 2 * ff, W,
+                                            hb_rowmap{m->moe_count, m->moe_list, cap, top, (long)2 * ff * W, 0, 0, 0}, E.experts));
+        hipLaunchKernelGGL(k_hb_glu_clamp, dim3(ne, (ff + 1023) / 1024), dim3(256), 0, st, m->ff, m->moe_act, ff, E.limit, E.act_alpha,
+                           m->moe_sel, E.experts);
+        VOX_TRY(hb_gemm_tiles<HB_EPI_STORE>(st, m->moe_act, (long)ff, (const T*)E.w_down, nullptr, m->moe_out, (long)W, n, W, ff,
+                                            hb_rowmap{m->moe_count, m->moe_list, cap, 1, (long)W * ff, 0, 0, 0}, E.experts));
     }
     hipLaunchKernelGGL(k_hb_moe_combine, dim3(n), dim3(256), 0, st, cur, ldx, h2, (long)W, m->moe_out, m->moe_sel, m->moe_wgt, top, E.experts, W);
     if (E.shared_ff > 0) {
@@ -1921,8 +2076,10 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
     if (ok && m->any_shift) ok = hipMalloc((void**)&m->shift, 5 * R * W * 4) == hipSuccess;
     if (ok && m->max_top > 0) {
         const size_t ne = R * (size_t)m->max_top;
-        ok = hipMalloc((void**)&m->moe_z, R * (size_t)m->max_ne * 4) == hipSuccess && hipMalloc((void**)&m->moe_wgt, ne * 4) == hipSuccess &&
-             hipMalloc((void**)&m->moe_sel, ne * 4) == hipSuccess && hipMalloc((void**)&m->moe_act, R * (size_t)(m->max_eff > 0 ? m->max_eff : 1) * 4) == hipSuccess &&
+        ok = hipMalloc((void**)&m->moe_wgt, ne * 4) == hipSuccess &&
+             hipMalloc((void**)&m->moe_sel, ne * 4) == hipSuccess &&
+             hipMalloc((void**)&m->moe_act, (R > HB_MOE_GEMV_ROWS * (size_t)(m->max_top + 1) ? R : HB_MOE_GEMV_ROWS * (size_t)(m->max_top + 1)) *
+                                                (size_t)(m->max_eff > 0 ? m->max_eff : 1) * 4) == hipSuccess &&
              hipMalloc((void**)&m->moe_out, ne * W * 4) == hipSuccess &&
              hipMalloc((void**)&m->moe_list, (size_t)(m->max_experts > 0 ? m->max_experts : 1) * R * 4) == hipSuccess &&
              hipMalloc((void**)&m->moe_count, (size_t)(m->max_experts > 0 ? m->max_experts : 1) * 4) == hipSuccess;
@@ -1946,7 +2103,7 @@ void vox_hybrid_destroy(vox_hybrid* m) {
     if (!m) return;
     (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->h2); (void)hipFree(m->proj); (void)hipFree(m->mix);
     (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws); (void)hipFree(m->shift);
-    (void)hipFree(m->moe_z); (void)hipFree(m->moe_wgt); (void)hipFree(m->moe_sel); (void)hipFree(m->moe_act); (void)hipFree(m->moe_out);
+    (void)hipFree(m->moe_wgt); (void)hipFree(m->moe_sel); (void)hipFree(m->moe_act); (void)hipFree(m->moe_out);
     (void)hipFree(m->moe_list); (void)hipFree(m->moe_count);
     delete m;
 }

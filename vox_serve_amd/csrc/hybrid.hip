@@ -151,16 +151,37 @@ __global__ __launch_bounds__(256) void k_hb_rms_groups(const float* x, long ldx,
                                                        float* y2, long ldy, int W, int groups, float eps) {
     const int r = blockIdx.x, src = rows ? rows[r] : r, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const int Wg = W / groups;
-    for (int g = wv; g < groups; g += 4) {
+    // 16-byte requests when every slice and row starts on one (a property of the sizes, not of the step); the lane-strided order of
+    // the scalar form otherwise
+    const bool vec = (Wg % 4 == 0) && (ldx % 4 == 0) && (ldy % 4 == 0) && (((size_t)x | (size_t)y1 | (size_t)w1 | (size_t)y2 | (size_t)w2) & 15) == 0;
+    for (int g = wv + 4 * blockIdx.y; g < groups; g += 4 * gridDim.y) {
         const float* xr = x + (size_t)src * ldx + (size_t)g * Wg;
         float ss = 0.f;
-        for (int i = lane; i < Wg; i += 64) ss = fmaf(xr[i], xr[i], ss);
+        if (vec) {
+            for (int i = lane * 4; i < Wg; i += 256) {
+                const float4 v = *(const float4*)(xr + i);
+                ss = fmaf(v.x, v.x, ss); ss = fmaf(v.y, v.y, ss); ss = fmaf(v.z, v.z, ss); ss = fmaf(v.w, v.w, ss);
+            }
+        } else {
+            for (int i = lane; i < Wg; i += 64) ss = fmaf(xr[i], xr[i], ss);
+        }
         ss = hb_wave_sum(ss);
         const float inv = 1.0f / sqrtf(ss / (float)Wg + eps);
-        for (int i = lane; i < Wg; i += 64) {
-            const float v = xr[i] * inv;
-            y1[(size_t)r * ldy + g * Wg + i] = v * w1[g * Wg + i];
-            if (w2) y2[(size_t)r * ldy + g * Wg + i] = v * w2[g * Wg + i];
+        if (vec) {
+            for (int i = lane * 4; i < Wg; i += 256) {
+                const float4 v = *(const float4*)(xr + i), a = *(const float4*)(w1 + g * Wg + i);
+                *(float4*)(y1 + (size_t)r * ldy + g * Wg + i) = make_float4(v.x * inv * a.x, v.y * inv * a.y, v.z * inv * a.z, v.w * inv * a.w);
+                if (w2) {
+                    const float4 b2 = *(const float4*)(w2 + g * Wg + i);
+                    *(float4*)(y2 + (size_t)r * ldy + g * Wg + i) = make_float4(v.x * inv * b2.x, v.y * inv * b2.y, v.z * inv * b2.z, v.w * inv * b2.w);
+                }
+            }
+        } else {
+            for (int i = lane; i < Wg; i += 64) {
+                const float v = xr[i] * inv;
+                y1[(size_t)r * ldy + g * Wg + i] = v * w1[g * Wg + i];
+                if (w2) y2[(size_t)r * ldy + g * Wg + i] = v * w2[g * Wg + i];
+            }
         }
     }
 }
@@ -942,7 +963,7 @@ __global__ __launch_bounds__(256) void k_hb_shift_mix(const float* h, long ldh, 
     const int row = blockIdx.x;
     const int r = row_req[row], rs = req_rows[r];
     const float* prev = row > rs ? h + (size_t)(row - 1) * ldh : (pos[row] == 0 ? nullptr : state + (size_t)req_state[r] * per_slot + prev_off);
-    for (int i = threadIdx.x; i < W; i += 256) {
+    for (int i = blockIdx.y * 256 + threadIdx.x; i < W; i += 256 * gridDim.y) {
         const float x = h[(size_t)row * ldh + i], d = (prev ? prev[i] : 0.f) - x;
 #pragma unroll
         for (int s2 = 0; s2 < 5; ++s2) mixes[(size_t)s2 * rows_stride + (size_t)row * W + i] = x + d * mu[(size_t)s2 * W + i];
@@ -1472,47 +1493,53 @@ __global__ __launch_bounds__(64) void k_hb_attn_merge(const float* part, int nse
 }
 
 // ---- routed feed-forward --------------------------------------------------------------------------------------------------
-// One wave per row: router logits z_j = router[j] . h in fp32 (lane-strided sums and a butterfly: an order fixed by the width, the
-// same for every step shape), s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first
+// One block per row: router logits z_j = router[j] . h in fp32 (lane-strided sums over four waves and a butterfly: an order fixed by
+// the width, the same for every step shape), then one wave: s = softmax(z) over all nE router outputs, choice = s + correction, the `top` largest choices (first
 // index wins a tie) in descending order; weights = their s / (sum + 1e-20).  sel[row*top + k] = router output index, wgt likewise.
-__global__ __launch_bounds__(64) void k_hb_moe_router(const float* h, long ldh, const float* router, const float* corr, int W, int nE, int top,
-                                                      int* sel, float* wgt) {
+__global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh, const float* router, const float* corr, int W, int nE, int top,
+                                                       int* sel, float* wgt) {
     extern __shared__ float sm[];
     float* sc = sm;                    // [nE] logits, then scores
     float* ch = sm + nE;               // [nE] choice values
     int* pick = (int*)(sm + 2 * nE);   // [top]
-    const int row = blockIdx.x, lane = threadIdx.x;
+    float* part = sm + 2 * nE + top;   // [4][nE] the waves' partial logits
+    const int row = blockIdx.x, lane = threadIdx.x & 63, wv = threadIdx.x >> 6;
     const float* x = h + (size_t)row * ldh;
     const bool vec = (W % 4 == 0) && (ldh % 4 == 0) && ((((size_t)h) & 15) == 0) && ((((size_t)router) & 15) == 0);
-    for (int j0 = 0; j0 < nE; j0 += 4) {
-        float acc[4] = {0.f, 0.f, 0.f, 0.f};
-        const float* r[4];
+    // wave w sums the k-chunks w, w + 4, ... (64 lanes x 4 values, or 64 values); a logit = the four waves' sums added in wave order
+    for (int j0 = 0; j0 < nE; j0 += 8) {
+        float acc[8];
+        const float* r[8];
 #pragma unroll
-        for (int j = 0; j < 4; ++j) r[j] = router + (size_t)(j0 + j < nE ? j0 + j : nE - 1) * W;
+        for (int j = 0; j < 8; ++j) { acc[j] = 0.f; r[j] = router + (size_t)(j0 + j < nE ? j0 + j : nE - 1) * W; }
         if (vec) {
-            for (int k = lane * 4; k < W; k += 256) {
+            for (int k = (wv * 64 + lane) * 4; k < W; k += 1024) {
                 const float4 xv = *(const float4*)(x + k);
 #pragma unroll
-                for (int j = 0; j < 4; ++j) {
+                for (int j = 0; j < 8; ++j) {
                     const float4 rv = *(const float4*)(r[j] + k);
                     acc[j] = fmaf(rv.x, xv.x, acc[j]); acc[j] = fmaf(rv.y, xv.y, acc[j]);
                     acc[j] = fmaf(rv.z, xv.z, acc[j]); acc[j] = fmaf(rv.w, xv.w, acc[j]);
                 }
             }
         } else {
-            for (int k = lane; k < W; k += 64) {
+            for (int k = wv * 64 + lane; k < W; k += 256) {
                 const float xv = x[k];
 #pragma unroll
-                for (int j = 0; j < 4; ++j) acc[j] = fmaf(r[j][k], xv, acc[j]);
+                for (int j = 0; j < 8; ++j) acc[j] = fmaf(r[j][k], xv, acc[j]);
             }
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
+        for (int j = 0; j < 8; ++j) {
             const float v = hb_wave_sum(acc[j]);
-            if (lane == 0 && j0 + j < nE) sc[j0 + j] = v;
+            if (lane == 0 && j0 + j < nE) part[wv * nE + j0 + j] = v;
         }
     }
     __syncthreads();
+    if (wv != 0) return;
+    for (int i = lane; i < nE; i += 64) sc[i] = ((part[i] + part[nE + i]) + part[2 * nE + i]) + part[3 * nE + i];
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
     float mx = -INFINITY;
     for (int i = lane; i < nE; i += 64) mx = fmaxf(mx, sc[i]);
     mx = hb_wave_max(mx);
@@ -1528,7 +1555,9 @@ __global__ __launch_bounds__(64) void k_hb_moe_router(const float* h, long ldh, 
         sc[i] = v;
         ch[i] = v + (corr ? corr[i] : 0.f);
     }
-    __syncthreads();
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    __builtin_amdgcn_wave_barrier();
+    // one wave from here on: every lane follows the same picks; lane 0 retires a pick in LDS before the next search reads it
     float wsum = 0.f;
     for (int k = 0; k < top; ++k) {
         float best = -INFINITY;
@@ -1544,10 +1573,13 @@ __global__ __launch_bounds__(64) void k_hb_moe_router(const float* h, long ldh, 
             if (ov > best || (ov == best && oi < at)) { best = ov; at = oi; }
         }
         if (at == 0x7fffffff) at = 0;
-        wsum += sc[at];
-        __syncthreads();
-        if (lane == 0) { pick[k] = at; ch[at] = -INFINITY; }
-        __syncthreads();
+        const float sv = sc[at];
+        wsum += sv;
+        if (lane == (k & 63)) { pick[k] = at; }
+        __builtin_amdgcn_wave_barrier();
+        if (lane == 0) ch[at] = -INFINITY;
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+        __builtin_amdgcn_wave_barrier();
     }
     const float den = wsum + 1e-20f;
     for (int k = lane; k < top; k += 64) {
@@ -1778,7 +1810,8 @@ static void hb_norm(const vox_hybrid* m, hipStream_t st, int n, const float* x, 
                     const float* w2, float* y2, long ldy) {
     const vox_hybrid_config& c = m->cfg;
     if (c.norm_kind == VOX_NORM_RMS_GROUPS) {
-        hipLaunchKernelGGL(k_hb_rms_groups, dim3(n), dim3(256), 0, st, x, ldx, rows, w1, y1, w2, y2, ldy, c.width, c.norm_groups, c.eps);
+        hipLaunchKernelGGL(k_hb_rms_groups, dim3(n, (c.norm_groups + 3) / 4 < 8 ? (c.norm_groups + 3) / 4 : 8), dim3(256), 0, st, x, ldx, rows, w1, y1,
+                           w2, y2, ldy, c.width, c.norm_groups, c.eps);
     } else {
         hb_layernorm(st, n, x, ldx, rows, w1, y1, ldy, c.width, c.eps);
         if (w2) hb_layernorm(st, n, x, ldx, rows, w2, y2, ldy, c.width, c.eps);
@@ -1803,7 +1836,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         if (!hn) { hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, nullptr, nullptr, (long)W); hn = m->h; }
         const int HD = L.heads * L.dim;
         const long per_slot = (long)HD * L.dim + W, rows_stride = (long)c.max_rows * W;
-        hipLaunchKernelGGL(k_hb_shift_mix, dim3(n), dim3(256), 0, st, hn, (long)W, L.shift_mu, m->shift, rows_stride, state, per_slot,
+        hipLaunchKernelGGL(k_hb_shift_mix, dim3(n, n <= 64 ? (W + 255) / 256 : 1), dim3(256), 0, st, hn, (long)W, L.shift_mu, m->shift, rows_stride, state, per_slot,
                            (long)HD * L.dim, io->pos, io->row_req, io->req_rows, io->req_state, W);
         const T* wi = (const T*)L.w_in;
         // r, k, v, g: four products of one shape, each on its own mix, in one launch
@@ -1902,7 +1935,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
 template <typename T>
 static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const float* h2, float* cur, long ldx, int n) {
     const int W = m->cfg.width, nE = E.experts + E.identity, top = E.top, ne = n * top, ff = E.ff;
-    hipLaunchKernelGGL(k_hb_moe_router, dim3(n), dim3(64), (size_t)(2 * nE + top) * 4, st, h2, (long)W, E.router, E.correction, W, nE, top,
+    hipLaunchKernelGGL(k_hb_moe_router, dim3(n), dim3(256), (size_t)(6 * nE + top) * 4, st, h2, (long)W, E.router, E.correction, W, nE, top,
                        m->moe_sel, m->moe_wgt);
     if (n <= HB_MOE_GEMV_ROWS) {
         const int per = top + (E.shared_ff > 0 ? 1 : 0), maxf = ff > E.shared_ff ? ff : E.shared_ff;

@@ -155,6 +155,34 @@ def test_mixed_batch_matches_each_alone():
         d.close()
 
 
+def test_long_step_shared_by_requests():
+    """A step of more than 64 rows (the recurrent unit cuts every request's rows into chunks that run side by side, the routed
+    feed-forward runs expert by expert) shared by a long portion, a short one, and single decoded tokens."""
+    cfg = stack()
+    S = F.random_checkpoint(cfg, seed=61, identity_bias=0.1)
+    seqs = {"a": tokens(150, 64, 62), "b": tokens(40, 64, 63), "c": tokens(12, 64, 64)}
+    want = {k: FR.forward(cfg, S, v) for k, v in seqs.items()}
+    d = U.Driver(cfg, S, pages=64)
+    try:
+        got = {k: [] for k in seqs}
+        steps = [[("c", 0, 10)], [("a", 0, 97), ("b", 0, 3), ("c", 10, 11)], [("a", 97, 98), ("b", 3, 40), ("c", 11, 12)], [("a", 98, 150)]]
+        for st in steps:
+            out = d.feed([(k, seqs[k][lo:hi]) for k, lo, hi in st])
+            for k, lg in out.items():
+                got[k].append(lg)
+        for k in seqs:
+            assert U.rel_err(torch.cat(got[k], 0), want[k]) < F32_BAR, k
+    finally:
+        d.close()
+
+
+def test_identity_outputs_only():
+    """A router with identity outputs only and no shared expert: the feed-forward adds the normed input itself."""
+    cfg = F.config([F.rglru(mlp=F.moe(experts=0, identity=2, top=1, shared=None)), F.parallel(mlp=F.moe(experts=0, identity=3, top=2, shared=(6, 1.0)))])
+    S = F.random_checkpoint(cfg, seed=65)
+    check(cfg, S, tokens(30, 40, 66), [20, 2])
+
+
 def test_pages_and_slots_are_reused():
     """6 pages and 2 state slots serve six requests, two at a time: stale K / V, recurrent state, convolution history or a
     previous owner's last input must not leak into the next owner."""

@@ -216,14 +216,24 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
         for (int j = 0; j < NT; ++j) acc[i][j] = hb_f32x4{0.f, 0.f, 0.f, 0.f};
     const bool a_vec = (K % 4 == 0) && (lda % 4 == 0) && ((((size_t)A) & 15) == 0);
     const bool w_vec = (K % 8 == 0) && ((((size_t)Wt) & 15) == 0);
-    for (int k0 = 0; k0 < K; k0 += BK) {
-        // A tile: BM x 64 fp32 -> bf16
-        for (int idx = tid; idx < BM * 16; idx += 256) {
-            const int r = idx >> 4, c = (idx & 15) * 4;
-            const int gm = m0 + r, gk = k0 + c;
+    // the next k-tile's global requests are issued before the current tile's products and land in registers meanwhile
+    constexpr int NA = BM * 16 / 256;
+    float4 ra[NA];
+    uint4 rw[2];
+    const float* arow[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        const int gm = m0 + ((tid + i * 256) >> 4);
+        arow[i] = gm < M ? A + (size_t)(lst ? lst[gm] / rm.a_div : gm) * lda : nullptr;
+    }
+    auto fetch = [&](int k0) {
+        // A tile: BM x 64 fp32
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const int gk = k0 + ((tid + i * 256) & 15) * 4;
             float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (gm < M) {
-                const float* p = A + (size_t)(lst ? lst[gm] / rm.a_div : gm) * lda + gk;
+            if (arow[i]) {
+                const float* p = arow[i] + gk;
                 if (a_vec && gk + 3 < K) v = *(const float4*)p;
                 else {
                     if (gk < K) v.x = p[0];
@@ -232,15 +242,13 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
                     if (gk + 3 < K) v.w = p[3];
                 }
             }
-            uint2 o;
-            o.x = pack_bf2(v.x, v.y);
-            o.y = pack_bf2(v.z, v.w);
-            *(uint2*)(As + r * LD + c) = o;
+            ra[i] = v;
         }
         // W tile: 64 x 64 bf16
-        for (int idx = tid; idx < 64 * 8; idx += 256) {
-            const int r = idx >> 3, c = (idx & 7) * 8;
-            const int gn = n0 + r, gk = k0 + c;
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = tid + i * 256;
+            const int gn = n0 + (idx >> 3), gk = k0 + (idx & 7) * 8;
             uint4 v = make_uint4(0, 0, 0, 0);
             if (gn < N) {
                 const bf16_t* p = Wt + (size_t)gn * K + gk;
@@ -253,9 +261,26 @@ __global__ __launch_bounds__(256) void k_hb_gemm_bf16(const float* A, long lda, 
                     v.z = t[4] | ((u32)t[5] << 16); v.w = t[6] | ((u32)t[7] << 16);
                 }
             }
-            *(uint4*)(Ws + r * LD + c) = v;
+            rw[i] = v;
+        }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += BK) {
+#pragma unroll
+        for (int i = 0; i < NA; ++i) {
+            const int idx = tid + i * 256;
+            uint2 o;
+            o.x = pack_bf2(ra[i].x, ra[i].y);
+            o.y = pack_bf2(ra[i].z, ra[i].w);
+            *(uint2*)(As + (idx >> 4) * LD + (idx & 15) * 4) = o;
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int idx = tid + i * 256;
+            *(uint4*)(Ws + (idx >> 3) * LD + (idx & 7) * 8) = rw[i];
         }
         __syncthreads();
+        if (k0 + BK < K) fetch(k0 + BK);
 #pragma unroll
         for (int ks = 0; ks < BK; ks += 32) {
             hb_bf16x8 af[MT], bfr[NT];
@@ -1940,8 +1965,9 @@ static int hb_moe(vox_hybrid* m, hipStream_t st, const vox_hybrid_moe& E, const 
     if (n <= HB_MOE_GEMV_ROWS) {
         const int per = top + (E.shared_ff > 0 ? 1 : 0), maxf = ff > E.shared_ff ? ff : E.shared_ff;
         const hb_moe_small q{m->moe_sel, m->moe_wgt, top, E.experts, ff, E.shared_ff, m->max_eff, E.limit, E.shared_limit, E.act_alpha};
-        hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((maxf + 3) / 4, n * per), dim3(256), 0, st, h2, (long)W, (const T*)E.w_gate_up,
-                           (const T*)E.shared_gate_up, m->moe_act, W, q);
+        if (maxf > 0 && per > 0 && (E.experts > 0 || E.shared_ff > 0))
+            hipLaunchKernelGGL((k_hb_moe_gate_up<T>), dim3((maxf + 3) / 4, n * per), dim3(256), 0, st, h2, (long)W, (const T*)E.w_gate_up,
+                               (const T*)E.shared_gate_up, m->moe_act, W, q);
         hipLaunchKernelGGL((k_hb_moe_down_combine<T>), dim3((W + 3) / 4, n), dim3(256), 0, st, h2, (long)W, (const T*)E.w_down,
                            (const T*)E.shared_down, m->moe_act, cur, ldx, W, q);
         return VOX_OK;

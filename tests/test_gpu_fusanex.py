@@ -327,6 +327,21 @@ def test_wide_sizes():
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_matrix_core_sizes(dtype):
+    """Sizes at which every product takes its matrix-core or 16-byte form (widths and inner sizes that are multiples of 32), with
+    prompt portions of 130 / 9 / 2 / 33 rows and decoding: the row-tile, tile and per-expert gathered forms against the same oracle."""
+    layers = [F.parallel(heads=8, kv_heads=2, dim=32, vdim=64, every=50, rheads=3, rdim=64, mlp=F.moe(experts=6, identity=1, top=3, ff=96, shared=(160, 1.0))),
+              F.rglru(width=512, blocks=4, conv=3, mlp=F.moe(experts=6, identity=1, top=3, ff=96, shared=(160, 1.0))),
+              F.parallel(heads=4, kv_heads=4, dim=64, vdim=32, every=64, rheads=6, rdim=32, mlp=F.moe(experts=4, identity=0, top=2, ff=128, shared=None))]
+    cfg = F.config(layers, width=384, vocab=500, groups=6, embed_scale=4.0)
+    S = F.random_checkpoint(cfg, seed=71, lora=32)
+    toks = tokens(190, 500, 72)
+    q = None if dtype == torch.float32 else 0.95
+    check(cfg, S, toks, [130, 9, 2, 33], dtype=dtype, quantile=q, page_size=64, pages=8, max_rows=192)
+    check(cfg, S, toks, [190], dtype=dtype, quantile=q, page_size=64, pages=8, max_rows=192)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_odd_sizes(dtype):
     """Sizes that defeat every vector path: width 18, key dims 10 / 5, value dims 6 / 7, 3 query heads per K/V head, matrix-state
     heads of 3 and 5 dims, gate blocks of 7 and 3 channels, a 37-entry vocabulary, expert widths 5 and 9, norm groups of 9 and 1."""

@@ -44,6 +44,30 @@ template <typename T> __device__ __forceinline__ float hb_operand(float v);
 template <> __device__ __forceinline__ float hb_operand<float>(float v) { return v; }
 template <> __device__ __forceinline__ float hb_operand<bf16_t>(float v) { return bfround(v); }
 
+// A lane-chunked dot product in k_hb_gemv's order: chunks of CH at lane*CH + 64*CH*i, then a butterfly.
+template <typename T>
+__device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, bool vec, int lane) {
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    float a = 0.f;
+    if (vec) {
+        for (int k = lane * CH; k < K; k += 64 * CH) {
+            float wv[CH];
+            if (sizeof(T) == 2) {
+                const uint4 u = *(const uint4*)(w + k);
+                wv[0] = bflo(u.x); wv[1] = bfhi(u.x); wv[2] = bflo(u.y); wv[3] = bfhi(u.y);
+                if (CH == 8) { wv[4] = bflo(u.z); wv[5] = bfhi(u.z); wv[6] = bflo(u.w); wv[7] = bfhi(u.w); }
+            } else {
+                const float4 u = *(const float4*)(w + k);
+                wv[0] = u.x; wv[1] = u.y; wv[2] = u.z; wv[3] = u.w;
+            }
+#pragma unroll
+            for (int i = 0; i < CH; ++i) a = fmaf(wv[i], hb_operand<T>(x[k + i]), a);
+        }
+    } else {
+        for (int k = lane; k < K; k += 64) a = fmaf(hb_ld(w + k), hb_operand<T>(x[k]), a);
+    }
+    return hb_wave_sum(a);
+}
 enum { HB_EPI_STORE = 0, HB_EPI_GELU = 1, HB_EPI_RESID = 2, HB_EPI_TANH = 3 };
 template <int EPI> __device__ __forceinline__ void hb_epilogue(float* c, float acc, float bias) {
     float v = acc + bias;
@@ -1002,7 +1026,8 @@ template <int DPW>
 __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(const float* proj, long ldp, float* out, long ldo, const float* bonus,
                                                                                 float* state, long per_slot, const float* h, long ldh, int W,
                                                                                 const int* req_rows, const int* req_state, const int* pos,
-                                                                                int H, int dim, int lora, int TT) {
+                                                                                int H, int dim, int lora, int TT, const float* head_w, float eps,
+                                                                                float out_scale) {
     extern __shared__ float sm[];
     const int nw = blockDim.x >> 6, dpad = nw * DPW;
     float* rsm = sm;                       // [TT][dpad]
@@ -1059,10 +1084,19 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(
             float* pt = part + flip * nw * 64;
             pt[w * 64 + lane] = o;
             __syncthreads();
-            if (w == 0 && ok) {
-                float sum = pt[lane];
-                for (int k = 1; k < nw; ++k) sum += pt[k * 64 + lane];
-                out[(size_t)(t0 + tt) * ldo + hd * dim + c] = sum;
+            if (w == 0) {
+                float sum = 0.f;
+                if (ok) {
+                    sum = pt[lane];
+                    for (int k = 1; k < nw; ++k) sum += pt[k * 64 + lane];
+                }
+                if (head_w) {
+                    // the block holds the whole head (dim <= 64): unit RMS, weight, silu gate and the mixer's scale here
+                    const float inv = 1.0f / sqrtf(hb_wave_sum(sum * sum) / (float)dim + eps);
+                    const float g = ok ? proj[(size_t)(t0 + tt) * ldp + 3 * HD + hd * dim + c] : 0.f;
+                    sum = sum * inv * (ok ? head_w[hd * dim + c] : 0.f) * (g * hb_sigmoid(g)) * out_scale;
+                }
+                if (ok) out[(size_t)(t0 + tt) * ldo + hd * dim + c] = sum;
             }
             flip ^= 1;
         }
@@ -1647,30 +1681,6 @@ __global__ __launch_bounds__(256) void k_hb_glu_clamp(const float* gu, float* y,
     }
 }
 // Few-row steps.  Entries per row: its `top` routed choices, then (shared_ff > 0) the shared expert.
-// A lane-chunked dot product in k_hb_gemv's order: chunks of CH at lane*CH + 64*CH*i, then a butterfly.
-template <typename T>
-__device__ __forceinline__ float hb_dot_wave(const T* w, const float* x, int K, bool vec, int lane) {
-    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
-    float a = 0.f;
-    if (vec) {
-        for (int k = lane * CH; k < K; k += 64 * CH) {
-            float wv[CH];
-            if (sizeof(T) == 2) {
-                const uint4 u = *(const uint4*)(w + k);
-                wv[0] = bflo(u.x); wv[1] = bfhi(u.x); wv[2] = bflo(u.y); wv[3] = bfhi(u.y);
-                if (CH == 8) { wv[4] = bflo(u.z); wv[5] = bfhi(u.z); wv[6] = bflo(u.w); wv[7] = bfhi(u.w); }
-            } else {
-                const float4 u = *(const float4*)(w + k);
-                wv[0] = u.x; wv[1] = u.y; wv[2] = u.z; wv[3] = u.w;
-            }
-#pragma unroll
-            for (int i = 0; i < CH; ++i) a = fmaf(wv[i], hb_operand<T>(x[k + i]), a);
-        }
-    } else {
-        for (int k = lane; k < K; k += 64) a = fmaf(hb_ld(w + k), hb_operand<T>(x[k]), a);
-    }
-    return hb_wave_sum(a);
-}
 struct hb_moe_small {
     const int* sel;
     const float* wgt;
@@ -1874,10 +1884,15 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         const int tt = 4096 / dpad >= 16 ? 16 : (4096 / dpad >= 1 ? 4096 / dpad : 1);
         auto kern = dpw == 16 ? k_hb_shift_decay_scan<16> : (dpw == 32 ? k_hb_shift_decay_scan<32> : k_hb_shift_decay_scan<64>);
         const size_t lds = (size_t)(3 * tt * dpad + tt * 64 + 2 * nwv * 64) * 4;
+        // few-row steps with heads of at most 64 dims (one block holds a head): the scan also applies the head norm, the gate and the
+        // scale (per token that is a reduction inside the sequential loop, which long portions leave to a launch of its own)
+        const bool fused_norm = L.dim <= 64 && n <= HB_MOE_GEMV_ROWS;
         hipLaunchKernelGGL(kern, dim3(n_req, L.heads, (L.dim + 63) / 64), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
-                           state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt);
-        hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj, 3 * HD,
-                           (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
+                           state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,
+                           fused_norm ? L.head_norm : (const float*)nullptr, c.eps, L.out_scale);
+        if (!fused_norm)
+            hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj, 3 * HD,
+                               (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
         return hb_gemm<T>(st, HB_EPI_RESID, m->mix, n_mix, (const T*)L.w_out, nullptr, cur, ldx, n, W, n_mix);
     }
     if (!hn && !(n == 1 && hb_try_norm_gemv<T>(m, st, HB_EPI_STORE, cur, ldx, nullptr, L.norm1, (const T*)L.w_in, L.b_in, m->proj, n_in, W))) {

@@ -10,7 +10,7 @@ gap = 0
 prev = None
 for r in rows:
     s, e = int(r["Start_Timestamp"]), int(r["End_Timestamp"])
-    name = r["Kernel_Name"].split("(")[0].replace("void ", "")[:34]
+    name = r["Kernel_Name"].replace("(anonymous namespace)::", "").replace("void ", "").split("(")[0][:44]
     d[(name, int(r["Grid_Size_X"]) // max(1, int(r["Workgroup_Size_X"])), r["Grid_Size_Y"], r["Grid_Size_Z"])].append(e - s)
     if prev is not None and 0 < s - prev < 50000:
         gap += s - prev
@@ -18,4 +18,4 @@ for r in rows:
 tot = sum(sum(v) for v in d.values())
 print(f"kernels {len(rows)}  busy {tot/1e6:.3f} ms  small-gaps {gap/1e6:.3f} ms")
 for k, v in sorted(d.items(), key=lambda kv: -sum(kv[1]))[:28]:
-    print(f"{k[0]:36s} grid {k[1]:5d}x{k[2]}x{k[3]:3s} n={len(v):5d} avg {sum(v)/len(v)/1e3:7.2f} us  tot {sum(v)/1e6:7.3f} ms  {100*sum(v)/tot:5.1f}%")
+    print(f"{k[0]:46s} grid {k[1]:5d}x{k[2]}x{k[3]:3s} n={len(v):5d} avg {sum(v)/len(v)/1e3:7.2f} us  tot {sum(v)/1e6:7.3f} ms  {100*sum(v)/tot:5.1f}%")

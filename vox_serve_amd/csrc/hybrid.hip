@@ -1022,12 +1022,19 @@ __global__ __launch_bounds__(256) void k_hb_shift_mix(const float* h, long ldh, 
 // Block = (request, head, 64 value columns); wave w keeps DPW key dims of the state in registers for the whole portion.  Per
 // token: o = sum_i (S_i + bonus_i k_i v) r_i, then S_i <- decay_i S_i + k_i v; the waves' partial outputs are added in wave order.
 // Block (r, 0, 0) finally stores the request's last normed input behind the matrix state (the next step's h_prev).
+// Long portions run the request's rows in chunks of `chunk_len` side by side (mode 1, 2 with k_hb_shift_decay_carry between them):
+//   mode 0  the whole portion from the slot's state, outputs, state and previous input stored (few-row steps)
+//   mode 1  chunk z from a zero state, no outputs: its final state B and the product A of its decays go to the workspace
+//   mode 2  chunk z replayed from its carry (left in the workspace by the carry kernel), outputs written
+// Workspace entry of chunk k of request r: index rs / chunk_len + r + k (unique: the chunks of the requests before r number at most
+// rs / chunk_len + r), [H][dim*dim + dim] floats each.
+enum { HB_SCAN_WHOLE = 0, HB_SCAN_REDUCE = 1, HB_SCAN_REPLAY = 2 };
 template <int DPW>
 __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(const float* proj, long ldp, float* out, long ldo, const float* bonus,
                                                                                 float* state, long per_slot, const float* h, long ldh, int W,
                                                                                 const int* req_rows, const int* req_state, const int* pos,
                                                                                 int H, int dim, int lora, int TT, const float* head_w, float eps,
-                                                                                float out_scale) {
+                                                                                float out_scale, int mode, int chunk_len, float* ws) {
     extern __shared__ float sm[];
     const int nw = blockDim.x >> 6, dpad = nw * DPW;
     float* rsm = sm;                       // [TT][dpad]
@@ -1035,18 +1042,24 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(
     float* wsm = ksm + TT * dpad;          // [TT][dpad]
     float* vsm = wsm + TT * dpad;          // [TT][64]
     float* part = vsm + TT * 64;           // [2][nw][64]
-    const int r = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = blockIdx.z * 64 + lane;
+    const int vt = (dim + 63) >> 6, chunk = mode == HB_SCAN_WHOLE ? 0 : blockIdx.z / vt, tile = mode == HB_SCAN_WHOLE ? blockIdx.z : blockIdx.z % vt;
+    const int r = blockIdx.x, hd = blockIdx.y, lane = threadIdx.x & 63, w = threadIdx.x >> 6, c = tile * 64 + lane;
     const int d0 = w * DPW;
-    const int rs = req_rows[r], re = req_rows[r + 1];
-    if (rs >= re) return;
-    const bool ok = c < dim, fresh = pos[rs] == 0;
+    const int rs0 = req_rows[r], re0 = req_rows[r + 1];
+    const int rs = mode == HB_SCAN_WHOLE ? rs0 : rs0 + chunk * chunk_len;
+    if (rs >= re0) return;
+    const int re = mode == HB_SCAN_WHOLE || rs + chunk_len > re0 ? re0 : rs + chunk_len;
+    const bool ok = c < dim, fresh = pos[rs0] == 0;
     float* slot = state + (size_t)req_state[r] * per_slot;
     float* St = slot + (size_t)hd * dim * dim;
-    float S[DPW], u[DPW];
+    if (mode != HB_SCAN_WHOLE) St = ws + ((size_t)(rs0 / chunk_len + r + chunk) * H + hd) * ((size_t)dim * dim + dim);
+    const bool load = mode == HB_SCAN_REPLAY || (mode == HB_SCAN_WHOLE && !fresh);
+    float S[DPW], u[DPW], A[DPW];
 #pragma unroll
     for (int i = 0; i < DPW; ++i) {
-        S[i] = (ok && !fresh && d0 + i < dim) ? St[(size_t)(d0 + i) * dim + c] : 0.f;
+        S[i] = (ok && load && d0 + i < dim) ? St[(size_t)(d0 + i) * dim + c] : 0.f;
         u[i] = d0 + i < dim ? bonus[hd * dim + d0 + i] : 0.f;
+        A[i] = 1.f;
     }
     const int HD = H * dim, off_d = 4 * HD + lora;
     int flip = 0;
@@ -1065,10 +1078,23 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(
             rsm[idx] = rv; ksm[idx] = kv; wsm[idx] = wv;
         }
         for (int idx = threadIdx.x; idx < nt * 64; idx += blockDim.x) {
-            const int tt = idx >> 6, cc = blockIdx.z * 64 + (idx & 63);
+            const int tt = idx >> 6, cc = tile * 64 + (idx & 63);
             vsm[idx] = cc < dim ? proj[(size_t)(t0 + tt) * ldp + 2 * HD + hd * dim + cc] : 0.f;
         }
         __syncthreads();
+        if (mode == HB_SCAN_REDUCE) {
+            for (int tt = 0; tt < nt; ++tt) {
+                const float v = vsm[tt * 64 + lane];
+                const float* kt = ksm + tt * dpad + d0;
+                const float* wt = wsm + tt * dpad + d0;
+#pragma unroll
+                for (int i = 0; i < DPW; ++i) {
+                    S[i] = wt[i] * S[i] + kt[i] * v;
+                    A[i] *= wt[i];
+                }
+            }
+            continue;
+        }
         for (int tt = 0; tt < nt; ++tt) {
             const float v = vsm[tt * 64 + lane];
             const float* rt = rsm + tt * dpad + d0;
@@ -1101,13 +1127,46 @@ __global__ __launch_bounds__(64 * HB_SCAN_MAX_WAVES) void k_hb_shift_decay_scan(
             flip ^= 1;
         }
     }
-    if (ok)
+    if (mode == HB_SCAN_REPLAY) return;
 #pragma unroll
-        for (int i = 0; i < DPW; ++i)
-            if (d0 + i < dim) St[(size_t)(d0 + i) * dim + c] = S[i];
-    if (hd == 0 && blockIdx.z == 0) {
+    for (int i = 0; i < DPW; ++i)
+        if (d0 + i < dim) {
+            if (ok) St[(size_t)(d0 + i) * dim + c] = S[i];
+            if (mode == HB_SCAN_REDUCE && tile == 0 && lane == 0) St[(size_t)dim * dim + d0 + i] = A[i];
+        }
+    if (mode == HB_SCAN_WHOLE && hd == 0 && blockIdx.z == 0) {
         float* prev = slot + (size_t)H * dim * dim;
         for (int i = threadIdx.x; i < W; i += blockDim.x) prev[i] = h[(size_t)(re - 1) * ldh + i];
+    }
+}
+// Between the two chunked passes: the slot's state is pushed through the request's chunks in order, S <- A_k S + B_k; every chunk's
+// workspace entry receives its carry-in in place of B_k, the slot the final state and the request's last normed input.
+__global__ __launch_bounds__(256) void k_hb_shift_decay_carry(float* ws, float* state, long per_slot, const float* h, long ldh, int W,
+                                                              const int* req_rows, const int* req_state, const int* pos, int H, int dim,
+                                                              int chunk_len) {
+    const int r = blockIdx.x, hd = blockIdx.y;
+    const int rs = req_rows[r], re = req_rows[r + 1];
+    if (rs >= re) return;
+    const int nc = (re - rs + chunk_len - 1) / chunk_len;
+    const bool fresh = pos[rs] == 0;
+    float* slot = state + (size_t)req_state[r] * per_slot;
+    float* St = slot + (size_t)hd * dim * dim;
+    const size_t per = (size_t)dim * dim + dim;
+    float* w0 = ws + ((size_t)(rs / chunk_len + r) * H + hd) * per;
+    for (int e = threadIdx.x; e < dim * dim; e += 256) {
+        const int kd = e / dim;
+        float S = fresh ? 0.f : St[e];
+        for (int k = 0; k < nc; ++k) {
+            float* wk = w0 + (size_t)k * H * per;
+            const float B = wk[e], A = wk[(size_t)dim * dim + kd];
+            wk[e] = S;
+            S = A * S + B;
+        }
+        St[e] = S;
+    }
+    if (hd == 0) {
+        float* prev = slot + (size_t)H * dim * dim;
+        for (int i = threadIdx.x; i < W; i += 256) prev[i] = h[(size_t)(re - 1) * ldh + i];
     }
 }
 
@@ -1800,6 +1859,7 @@ __global__ void k_hb_feedback(const int* out_ids, int* input_ids, uint64_t* rng,
 }  // namespace
 
 #define HB_MOE_GEMV_ROWS 8    // steps of at most this many rows run the routed feed-forward entry by entry
+#define HB_SCAN_CHUNK 64       // rows per chunk of the chunked matrix-state scan; steps of more rows take that form
 #define HB_LRU_SEQ_ROWS 64    // steps of at most this many rows run the gated linear recurrent unit token by token
 
 struct vox_hybrid {
@@ -1811,6 +1871,8 @@ struct vox_hybrid {
     vox_hybrid_weights w;
     float *xa = nullptr, *xb = nullptr, *h = nullptr, *h2 = nullptr, *proj = nullptr, *mix = nullptr, *ff = nullptr, *hout = nullptr;
     float *shift = nullptr;                 // [5][max_rows][width]: token-shift mixes
+    float *scan_ws = nullptr;               // chunk states and decay products of the chunked matrix-state scan
+    size_t scan_ws_floats = 0;
     float *moe_wgt = nullptr, *moe_act = nullptr, *moe_out = nullptr;
     int *moe_sel = nullptr, *moe_list = nullptr, *moe_count = nullptr;
     bf16_t* logits16 = nullptr;
@@ -1887,9 +1949,24 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         // few-row steps with heads of at most 64 dims (one block holds a head): the scan also applies the head norm, the gate and the
         // scale (per token that is a reduction inside the sequential loop, which long portions leave to a launch of its own)
         const bool fused_norm = L.dim <= 64 && n <= HB_MOE_GEMV_ROWS;
-        hipLaunchKernelGGL(kern, dim3(n_req, L.heads, (L.dim + 63) / 64), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
-                           state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,
-                           fused_norm ? L.head_norm : (const float*)nullptr, c.eps, L.out_scale);
+        const int vt = (L.dim + 63) / 64;
+        if (n > HB_SCAN_CHUNK && m->scan_ws) {
+            // steps of many rows: every request's rows in chunks of HB_SCAN_CHUNK side by side — each chunk reduced from a zero state,
+            // the carries pushed through in order, each chunk replayed from its carry (rounding aside the token-by-token form)
+            const int nch = (n + HB_SCAN_CHUNK - 1) / HB_SCAN_CHUNK;
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
+                               state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,
+                               (const float*)nullptr, c.eps, L.out_scale, (int)HB_SCAN_REDUCE, HB_SCAN_CHUNK, m->scan_ws);
+            hipLaunchKernelGGL(k_hb_shift_decay_carry, dim3(n_req, L.heads), dim3(256), 0, st, m->scan_ws, state, per_slot, hn, (long)W, W,
+                               io->req_rows, io->req_state, io->pos, L.heads, L.dim, HB_SCAN_CHUNK);
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
+                               state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,
+                               (const float*)nullptr, c.eps, L.out_scale, (int)HB_SCAN_REPLAY, HB_SCAN_CHUNK, m->scan_ws);
+        } else {
+            hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
+                               state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,
+                               fused_norm ? L.head_norm : (const float*)nullptr, c.eps, L.out_scale, (int)HB_SCAN_WHOLE, 0, (float*)nullptr);
+        }
         if (!fused_norm)
             hipLaunchKernelGGL(k_hb_head_norm, dim3(n, L.heads), dim3(64), 0, st, m->mix, (long)n_mix, L.head_norm, 1, m->proj, (long)n_proj, 3 * HD,
                                (int)HB_GATE_SILU, L.vdim, c.eps, L.out_scale);
@@ -2112,7 +2189,11 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
         if (n_proj > m->max_in) m->max_in = n_proj;
         if (L.heads * L.vdim > m->max_mix) m->max_mix = L.heads * L.vdim;
         if (L.ff > m->max_ff) m->max_ff = L.ff;
-        if (L.kind == VOX_MIXER_SHIFT_DECAY) m->any_shift = true;
+        if (L.kind == VOX_MIXER_SHIFT_DECAY) {
+            m->any_shift = true;
+            const size_t f = ((size_t)cfg->max_rows / HB_SCAN_CHUNK + cfg->max_batch + 1) * L.heads * ((size_t)L.dim * L.dim + L.dim);
+            if (f > m->scan_ws_floats) m->scan_ws_floats = f;
+        }
         if (L.moe) {
             const vox_hybrid_moe& E = *L.moe;
             if (E.experts + E.identity > m->max_ne) m->max_ne = E.experts + E.identity;
@@ -2148,6 +2229,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
               hipMalloc((void**)&m->hout, (size_t)cfg->max_out * W * 4) == hipSuccess &&
               hipMalloc((void**)&m->logits16, (size_t)cfg->max_batch * cfg->vocab * 2) == hipSuccess;
     if (ok && m->any_shift) ok = hipMalloc((void**)&m->shift, 5 * R * W * 4) == hipSuccess;
+    if (ok && m->scan_ws_floats && cfg->max_rows > HB_SCAN_CHUNK) ok = hipMalloc((void**)&m->scan_ws, m->scan_ws_floats * 4) == hipSuccess;
     if (ok && m->max_top > 0) {
         const size_t ne = R * (size_t)m->max_top;
         ok = hipMalloc((void**)&m->moe_wgt, ne * 4) == hipSuccess &&
@@ -2176,7 +2258,7 @@ int vox_hybrid_create(vox_ctx* ctx, const vox_hybrid_config* cfg, const vox_hybr
 void vox_hybrid_destroy(vox_hybrid* m) {
     if (!m) return;
     (void)hipFree(m->xa); (void)hipFree(m->xb); (void)hipFree(m->h); (void)hipFree(m->h2); (void)hipFree(m->proj); (void)hipFree(m->mix);
-    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws); (void)hipFree(m->shift);
+    (void)hipFree(m->ff); (void)hipFree(m->hout); (void)hipFree(m->logits16); (void)hipFree(m->attn_ws); (void)hipFree(m->shift); (void)hipFree(m->scan_ws);
     (void)hipFree(m->moe_wgt); (void)hipFree(m->moe_sel); (void)hipFree(m->moe_act); (void)hipFree(m->moe_out);
     (void)hipFree(m->moe_list); (void)hipFree(m->moe_count);
     delete m;

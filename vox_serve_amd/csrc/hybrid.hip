@@ -1018,6 +1018,78 @@ __global__ __launch_bounds__(256) void k_hb_shift_mix(const float* h, long ldh, 
         for (int s2 = 0; s2 < 5; ++s2) mixes[(size_t)s2 * rows_stride + (size_t)row * W + i] = x + d * mu[(size_t)s2 * W + i];
     }
 }
+// Few-row steps: the five mixes and their projections in one launch.  A wave per output column n of [r | k | v | g | bottleneck]:
+// its mix index is min(n / HD, 4); the operand x = h + (h_prev - h) * mu is formed in registers (the values k_hb_shift_mix stores),
+// summed in k_hb_gemv's order; the bottleneck's columns take tanh.
+template <typename T, int MR>
+__global__ __launch_bounds__(256) void k_hb_shift_gemv(const float* h, long ldh, const float* mu, const T* Wt, const float* bias, float* C, long ldc,
+                                                       const float* state, long per_slot, long prev_off, const int* pos, const int* row_req,
+                                                       const int* req_rows, const int* req_state, int M, int N, int HD, int W) {
+    const int lane = threadIdx.x & 63, n = blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (n >= N) return;
+    const int seg = n / HD < 4 ? n / HD : 4;
+    const float* mus = mu + (size_t)seg * W;
+    const T* wr = Wt + (size_t)n * W;
+    constexpr int CH = sizeof(T) == 2 ? 8 : 4;
+    const float* prev[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        prev[m] = nullptr;
+        if (m < M) {
+            const int r = row_req[m], rs = req_rows[r];
+            prev[m] = m > rs ? h + (size_t)(m - 1) * ldh : (pos[m] == 0 ? nullptr : state + (size_t)req_state[r] * per_slot + prev_off);
+        }
+    }
+    float acc[MR];
+#pragma unroll
+    for (int m = 0; m < MR; ++m) acc[m] = 0.f;
+    const bool vec = (W % CH == 0) && (ldh % 4 == 0) && ((per_slot | prev_off) % 4 == 0) &&
+                     ((((size_t)Wt) | ((size_t)h) | ((size_t)mu) | ((size_t)state)) & 15) == 0;
+    if (vec) {
+        for (int k = lane * CH; k < W; k += 64 * CH) {
+            float w[CH];
+            if (sizeof(T) == 2) {
+                const uint4 u = *(const uint4*)(wr + k);
+                w[0] = bflo(u.x); w[1] = bfhi(u.x); w[2] = bflo(u.y); w[3] = bfhi(u.y);
+                if (CH == 8) { w[4] = bflo(u.z); w[5] = bfhi(u.z); w[6] = bflo(u.w); w[7] = bfhi(u.w); }
+            } else {
+                const float4 u = *(const float4*)(wr + k);
+                w[0] = u.x; w[1] = u.y; w[2] = u.z; w[3] = u.w;
+            }
+#pragma unroll
+            for (int m = 0; m < MR; ++m) {
+                if (m >= M) break;
+#pragma unroll
+                for (int e = 0; e < CH; e += 4) {
+                    const float4 x4 = *(const float4*)(h + (size_t)m * ldh + k + e), m4 = *(const float4*)(mus + k + e);
+                    const float4 p4 = prev[m] ? *(const float4*)(prev[m] + k + e) : make_float4(0.f, 0.f, 0.f, 0.f);
+                    acc[m] = fmaf(w[e], hb_operand<T>(x4.x + (p4.x - x4.x) * m4.x), acc[m]);
+                    acc[m] = fmaf(w[e + 1], hb_operand<T>(x4.y + (p4.y - x4.y) * m4.y), acc[m]);
+                    acc[m] = fmaf(w[e + 2], hb_operand<T>(x4.z + (p4.z - x4.z) * m4.z), acc[m]);
+                    acc[m] = fmaf(w[e + 3], hb_operand<T>(x4.w + (p4.w - x4.w) * m4.w), acc[m]);
+                }
+            }
+        }
+    } else {
+        for (int k = lane; k < W; k += 64) {
+            const float w = hb_ld(wr + k);
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+                if (m < M) {
+                    const float x = h[(size_t)m * ldh + k], d = (prev[m] ? prev[m][k] : 0.f) - x;
+                    acc[m] = fmaf(w, hb_operand<T>(x + d * mus[k]), acc[m]);
+                }
+        }
+    }
+#pragma unroll
+    for (int m = 0; m < MR; ++m) {
+        const float sum = hb_wave_sum(acc[m]);
+        if (m < M && lane == 0) {
+            const float v = sum + (bias && seg < 4 ? bias[n] : 0.f);
+            C[(size_t)m * ldc + n] = seg == 4 ? tanhf(v) : v;
+        }
+    }
+}
 // proj row = [r | k | v | g (H*dim each) | decay bottleneck (lora) | decay pre-activation d (H*dim)]; decay = exp(-exp(d)).
 // Block = (request, head, 64 value columns); wave w keeps DPW key dims of the state in registers for the whole portion.  Per
 // token: o = sum_i (S_i + bonus_i k_i v) r_i, then S_i <- decay_i S_i + k_i v; the waves' partial outputs are added in wave order.
@@ -1933,13 +2005,26 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
         if (!hn) { hb_norm(m, st, n, cur, ldx, nullptr, L.norm1, m->h, nullptr, nullptr, (long)W); hn = m->h; }
         const int HD = L.heads * L.dim;
         const long per_slot = (long)HD * L.dim + W, rows_stride = (long)c.max_rows * W;
-        hipLaunchKernelGGL(k_hb_shift_mix, dim3(n, n <= 64 ? (W + 255) / 256 : 1), dim3(256), 0, st, hn, (long)W, L.shift_mu, m->shift, rows_stride, state, per_slot,
-                           (long)HD * L.dim, io->pos, io->row_req, io->req_rows, io->req_state, W);
         const T* wi = (const T*)L.w_in;
-        // r, k, v, g: four products of one shape, each on its own mix, in one launch
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->shift, W, wi, L.b_in, m->proj, n_proj, n, HD, W,
-                           hb_rowmap{nullptr, nullptr, 0, 1, (long)HD * W, rows_stride, (long)HD, (long)HD}, 4));
-        VOX_TRY(hb_gemm<T>(st, HB_EPI_TANH, m->shift + 4 * rows_stride, W, wi + (size_t)4 * HD * W, nullptr, m->proj + 4 * HD, n_proj, n, L.lora, W));
+        if (n == 1) {
+            // one row: mixes and the five projections in one launch
+            const dim3 g((4 * HD + L.lora + 3) / 4), b(256);
+#define HB_SHIFT(MR_) \
+    hipLaunchKernelGGL((k_hb_shift_gemv<T, MR_>), g, b, 0, st, hn, (long)W, L.shift_mu, wi, L.b_in, m->proj, (long)n_proj, state, per_slot, \
+                       (long)HD * L.dim, io->pos, io->row_req, io->req_rows, io->req_state, n, 4 * HD + L.lora, HD, W)
+            if (n == 1) HB_SHIFT(1);
+            else if (n == 2) HB_SHIFT(2);
+            else if (n <= 4) HB_SHIFT(4);
+            else HB_SHIFT(8);
+#undef HB_SHIFT
+        } else {
+            hipLaunchKernelGGL(k_hb_shift_mix, dim3(n, n <= 64 ? (W + 255) / 256 : 1), dim3(256), 0, st, hn, (long)W, L.shift_mu, m->shift, rows_stride,
+                               state, per_slot, (long)HD * L.dim, io->pos, io->row_req, io->req_rows, io->req_state, W);
+            // r, k, v, g: four products of one shape, each on its own mix, in one launch
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->shift, W, wi, L.b_in, m->proj, n_proj, n, HD, W,
+                               hb_rowmap{nullptr, nullptr, 0, 1, (long)HD * W, rows_stride, (long)HD, (long)HD}, 4));
+            VOX_TRY(hb_gemm<T>(st, HB_EPI_TANH, m->shift + 4 * rows_stride, W, wi + (size_t)4 * HD * W, nullptr, m->proj + 4 * HD, n_proj, n, L.lora, W));
+        }
         VOX_TRY(hb_gemm<T>(st, HB_EPI_STORE, m->proj + 4 * HD, n_proj, (const T*)L.w_decay2, L.decay0, m->proj + 4 * HD + L.lora, n_proj, n, HD, L.lora));
         const int dpw = L.dim <= 16 * HB_SCAN_MAX_WAVES ? 16 : (L.dim <= 32 * HB_SCAN_MAX_WAVES ? 32 : 64);
         const int nwv = (L.dim + dpw - 1) / dpw, dpad = nwv * dpw;

@@ -1225,7 +1225,7 @@ __global__ __launch_bounds__(256) void k_hb_shift_decay_carry(float* ws, float* 
     float* St = slot + (size_t)hd * dim * dim;
     const size_t per = (size_t)dim * dim + dim;
     float* w0 = ws + ((size_t)(rs / chunk_len + r) * H + hd) * per;
-    for (int e = threadIdx.x; e < dim * dim; e += 256) {
+    for (int e = blockIdx.z * 256 + threadIdx.x; e < dim * dim; e += 256 * gridDim.z) {
         const int kd = e / dim;
         float S = fresh ? 0.f : St[e];
         for (int k = 0; k < nc; ++k) {
@@ -1236,7 +1236,7 @@ __global__ __launch_bounds__(256) void k_hb_shift_decay_carry(float* ws, float* 
         }
         St[e] = S;
     }
-    if (hd == 0) {
+    if (hd == 0 && blockIdx.z == 0) {
         float* prev = slot + (size_t)H * dim * dim;
         for (int i = threadIdx.x; i < W; i += 256) prev[i] = h[(size_t)(re - 1) * ldh + i];
     }
@@ -2042,7 +2042,7 @@ static int hb_mixer(vox_hybrid* m, hipStream_t st, const vox_hybrid_io* io, cons
             hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
                                state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,
                                (const float*)nullptr, c.eps, L.out_scale, (int)HB_SCAN_REDUCE, HB_SCAN_CHUNK, m->scan_ws);
-            hipLaunchKernelGGL(k_hb_shift_decay_carry, dim3(n_req, L.heads), dim3(256), 0, st, m->scan_ws, state, per_slot, hn, (long)W, W,
+            hipLaunchKernelGGL(k_hb_shift_decay_carry, dim3(n_req, L.heads, (L.dim * L.dim + 255) / 256 < 64 ? (L.dim * L.dim + 255) / 256 : 64), dim3(256), 0, st, m->scan_ws, state, per_slot, hn, (long)W, W,
                                io->req_rows, io->req_state, io->pos, L.heads, L.dim, HB_SCAN_CHUNK);
             hipLaunchKernelGGL(kern, dim3(n_req, L.heads, vt * nch), dim3(64 * nwv), lds, st, m->proj, (long)n_proj, m->mix, (long)n_mix, L.bonus,
                                state, per_slot, hn, (long)W, W, io->req_rows, io->req_state, io->pos, L.heads, L.dim, L.lora, tt,

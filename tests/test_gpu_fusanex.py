@@ -308,6 +308,19 @@ def test_routed_choice_covers_every_expert_and_identity():
     check(cfg, S, toks, [50, 9, 2])
 
 
+def test_slow_decay_channels():
+    """Channels whose decay a is within 1e-4 of 1 (a very negative lambda): 1 - a^2 must not be formed by a subtraction of rounded
+    values — a relative error of 1e-7 in a would be one of 1e-3 in the input's weight sqrt(1 - a^2)."""
+    cfg = F.config([F.rglru(width=24, blocks=3, conv=2)], width=24)
+    S = F.random_checkpoint(cfg, seed=47)
+    lam = S["l0.mix.lam"].float()
+    lam[::2] = -11.0
+    S["l0.mix.lam"] = lam.to(torch.bfloat16)
+    toks = tokens(150, 40, 48)
+    check(cfg, S, toks, [150], bar=2e-5)
+    check(cfg, S, toks, [70, 3], bar=2e-5)
+
+
 def test_long_decoding():
     cfg = stack()
     S = F.random_checkpoint(cfg, seed=43)

@@ -916,8 +916,9 @@ __global__ __launch_bounds__(64) void k_hb_rglru_scan(const float* proj, long ld
             const int t = t0 + k < re ? t0 + k : re - 1;
             const float* pr = proj + (size_t)t * ldp;
             const float rg = hb_sigmoid(pr[off_r]), ig = hb_sigmoid(pr[off_i]);
-            a[k] = expf(-rec_scale * rg * sp);
-            b[k] = sqrtf(1.0f - a[k] * a[k]) * (ig * pr[2 * C + c]);
+            const float la = -rec_scale * rg * sp;
+            a[k] = expf(la);
+            b[k] = sqrtf(-expm1f(2.0f * la)) * (ig * pr[2 * C + c]);      // 1 - a^2 without the cancellation near a = 1
             y[k] = hb_gelu_tanh(pr[c]);
         }
 #pragma unroll
@@ -968,8 +969,9 @@ __global__ __launch_bounds__(1024) void k_hb_rglru_scan_chunked(float* proj, lon
             const int t = t0 + q < te ? t0 + q : te - 1;
             const float* pr = proj + (size_t)t * ldp;
             const float rg = hb_sigmoid(pr[off_r]), ig = hb_sigmoid(pr[off_i]);
-            a[q] = expf(-rec_scale * rg * sp);
-            b[q] = sqrtf(1.0f - a[q] * a[q]) * (ig * pr[2 * C + cc]);
+            const float la = -rec_scale * rg * sp;
+            a[q] = expf(la);
+            b[q] = sqrtf(-expm1f(2.0f * la)) * (ig * pr[2 * C + cc]);      // 1 - a^2 without the cancellation near a = 1
         }
 #pragma unroll
         for (int q = 0; q < 4; ++q)

@@ -1721,10 +1721,29 @@ __global__ __launch_bounds__(256) void k_hb_moe_router(const float* h, long ldh,
                 for (int j = 0; j < 8; ++j) acc[j] = fmaf(r[j][k], xv, acc[j]);
             }
         }
+        // eight sums over the wave with 10 exchanges instead of 48: each of the first three exchanges halves the values a lane
+        // carries (lanes with the partner bit clear keep the lower half and receive the partner's), three more finish the one left;
+        // the lane whose low three bits are clear ends up with the sum of value (bit 5, bit 4, bit 3 of its number)
+        {
+            const bool hi5 = lane & 32, hi4 = lane & 16, hi3 = lane & 8;
+            float b4[4], b2[2];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) {
-            const float v = hb_wave_sum(acc[j]);
-            if (lane == 0 && j0 + j < nE) part[wv * nE + j0 + j] = v;
+            for (int i = 0; i < 4; ++i) {
+                const float mine = hi5 ? acc[i + 4] : acc[i], give = hi5 ? acc[i] : acc[i + 4];
+                b4[i] = mine + __shfl_xor(give, 32, 64);
+            }
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float mine = hi4 ? b4[i + 2] : b4[i], give = hi4 ? b4[i] : b4[i + 2];
+                b2[i] = mine + __shfl_xor(give, 16, 64);
+            }
+            const float mine = hi3 ? b2[1] : b2[0], give = hi3 ? b2[0] : b2[1];
+            float v = mine + __shfl_xor(give, 8, 64);
+            v += __shfl_xor(v, 4, 64);
+            v += __shfl_xor(v, 2, 64);
+            v += __shfl_xor(v, 1, 64);
+            const int j = (hi5 ? 4 : 0) + (hi4 ? 2 : 0) + (hi3 ? 1 : 0);
+            if ((lane & 7) == 0 && j0 + j < nE) part[wv * nE + j0 + j] = v;
         }
     }
     __syncthreads();

@@ -412,6 +412,57 @@ def test_greedy_generation_through_the_scheduler():
         model.engine.close()
 
 
+def test_top_k_sampling_and_async_scheduling():
+    """Stochastic sampling goes through the library's sampler (every id is one of the oracle's five most likely continuations of
+    the request's own prefix; the same seed repeats the ids), and the pipelined scheduler loop generates the greedy ids."""
+    from vox_serve_amd.model import get_model_class
+    from vox_serve_amd.model.fusanex import config_from_dict
+    from vox_serve_amd.sampling import SamplingConfig
+    from vox_serve_amd.scheduler.base import Scheduler, encode_request
+    from vox_serve_amd.worker.base import ModelWorker
+    cfg = stack(sharp=False)
+    S = F.random_checkpoint(cfg, seed=91)
+    prompts = {"a": tokens(21, 64, 92), "b": tokens(9, 64, 93)}
+
+    def generate(sampling, n_new, greedy, async_scheduling):
+        model = get_model_class("fusanex")("fusanex-test", weights=S, config=config_from_dict(cfg), dtype=torch.float32, max_batch_size=2,
+                                           page_size=8, max_num_pages=32, max_seq_len=256, max_prefill_tokens=64, state_slots=2,
+                                           max_tokens=n_new, sampling=sampling)
+        worker = ModelWorker(model=model, max_batch_size=2, max_num_pages=32, page_size=8, seed=7, greedy=greedy, prefill_chunk_tokens=16)
+        sched = Scheduler(worker, max_batch_size=2, async_scheduling=async_scheduling)
+        seen = {}
+        orig = sched._prepare_requests
+
+        def spy():
+            orig()
+            for r in sched.active_requests:
+                seen[r.request_id] = r
+        sched._prepare_requests = spy
+        try:
+            for rid, p in prompts.items():
+                sched.transport.requests.put(encode_request(rid, " ".join(map(str, p)), is_streaming=False))
+            sched.run_until_idle(max_steps=400)
+            assert worker.empty_pages.qsize() == 32 and worker.empty_state_slots.qsize() == 2
+            return {rid: [int(t[0, 0]) for t in seen[rid].lm_output_tokens][:n_new] for rid in prompts}
+        finally:
+            model.engine.close()
+    first = generate(SamplingConfig(top_k=5, temperature=0.8, max_tokens=8), 8, False, False)
+    for rid, p in prompts.items():
+        assert len(first[rid]) == 8
+        seq = list(p)
+        for tok in first[rid]:
+            top = FR.forward(cfg, S, seq)[-1].topk(5).indices.tolist()
+            assert tok in top, (rid, tok, top)
+            seq.append(tok)
+    assert generate(SamplingConfig(top_k=5, temperature=0.8, max_tokens=8), 8, False, False) == first
+    got = generate(None, 7, True, True)
+    for rid, p in prompts.items():
+        seq = list(p)
+        for _ in range(7):
+            seq.append(int(FR.forward(cfg, S, seq)[-1].argmax()))
+        assert got[rid] == seq[len(p):], (rid, got[rid], seq[len(p):])
+
+
 def test_checkpoint_folder_through_the_registry(tmp_path):
     """config.json + model.safetensors in a folder: `load_checkpoint_dir` picks the design by the config's architecture."""
     import json
